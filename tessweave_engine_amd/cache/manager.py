@@ -25,7 +25,7 @@ class Sequence:
     """What the cache holds for one live request."""
 
     __slots__ = ("id", "state_slot", "tables", "computed", "cached", "promised", "budget", "closed",
-                 "block_keys", "key_namespace")
+                 "block_keys", "key_namespace", "steps")
 
     def __init__(self, seq_id, state_slot, n_groups):
         self.id = seq_id
@@ -36,6 +36,8 @@ class Sequence:
         self.promised = [0] * n_groups                 # pages promised to this request and not yet taken
         self.budget = [0] * n_groups                   # pages reserved at admission (0: grows on demand)
         self.closed = False
+        self.steps = 0                                 # steps that have run tokens of this request: a part that keeps its
+                                                       # state twice reads copy steps % 2 and writes the other
         self.block_keys = []                           # prefix-index keys of the first full blocks of its tokens, as far
         self.key_namespace = None                      # as they have been hashed (a request's tokens only grow)
 
@@ -76,8 +78,11 @@ class CacheManager:
         self.sequences: dict = {}
         self.dtype = dtype
         self.device = device
-        self.storage = []       # per group: tensor [slots, 2, pages, kv_heads, page_size, head_dim]
+        self.storage = []       # per group: tensor [slots, 2, pages, kv_heads, page_size, head_dim]; a group whose
+                                # values have a size of their own: (keys [slots, pages, kv_heads, page_size, head_dim],
+                                # values [slots, pages, kv_heads, page_size * value_dim])
         self.state = {}         # cache slot -> tensor [max_requests, *shape]
+        self.states = {}        # cache slot -> {name: tensor [max_requests, *shape]}
         if device is not None:
             self._allocate_storage()
 
@@ -92,21 +97,45 @@ class CacheManager:
                 raise ValueError("cache group too large")
             # Uninitialised on purpose (flow_engine/cache.py:22): a page's old
             # contents must never reach a result.
-            self.storage.append(torch.empty(shape, dtype=dtype, device=self.device))
+            if group.spec.value_dim is None:
+                self.storage.append(torch.empty(shape, dtype=dtype, device=self.device))
+            else:
+                keys = (shape[0],) + shape[2:]
+                values = keys[:-2] + (self.page_size * group.spec.value_dim,)
+                self.storage.append((torch.empty(keys, dtype=dtype, device=self.device),
+                                     torch.empty(values, dtype=dtype, device=self.device)))
         for slot in self.layout.state_slots:
             spec = self.layout.needs[slot].state
-            self.state[slot] = torch.zeros((self.max_requests,) + spec.shape,
-                                           dtype=getattr(torch, _STATE_DTYPES[spec.dtype]),
-                                           device=self.device)
+            self.state[slot] = self._state_tensor(spec)
+        for slot in self.layout.named_state_slots:
+            self.states[slot] = {name: self._state_tensor(spec) for name, spec in self.layout.needs[slot].states}
+
+    def _state_tensor(self, spec):
+        import torch
+        return torch.zeros((self.max_requests,) + spec.shape, dtype=getattr(torch, _STATE_DTYPES[spec.dtype]),
+                           device=self.device)
+
+    def _pool_tensors(self):
+        for t in self.storage:
+            yield from (t if isinstance(t, tuple) else (t,))
+
+    def _state_tensors(self):
+        yield from self.state.values()
+        for named in self.states.values():
+            yield from named.values()
 
     @property
     def allocated_bytes(self):
-        total = sum(t.numel() * t.element_size() for t in self.storage)
-        return total + sum(t.numel() * t.element_size() for t in self.state.values())
+        total = sum(t.numel() * t.element_size() for t in self._pool_tensors())
+        return total + sum(t.numel() * t.element_size() for t in self._state_tensors())
 
     def keys_values(self, cache_slot):
-        """(keys, values, group index) of CACHE_SLOT; each [pages, kv_heads, page_size, head_dim]."""
+        """(keys, values, group index) of CACHE_SLOT; each [pages, kv_heads, page_size, head_dim]. Where the
+        values have a size of their own they are [pages, kv_heads, page_size * value_dim]: how a page's values
+        are laid out is the business of the kernels that write and read them."""
         g, i = self.layout.slot_group[cache_slot]
+        if isinstance(self.storage[g], tuple):
+            return self.storage[g][0][i], self.storage[g][1][i], g
         return self.storage[g][i, 0], self.storage[g][i, 1], g
 
     # ---- requests ---------------------------------------------------------
@@ -117,7 +146,7 @@ class CacheManager:
             raise CapacityError("no free request slot")
         seq = Sequence(seq_id, self.free_state_slots.pop(), len(self.pools))
         self.sequences[seq_id] = seq
-        for slot, tensor in self.state.items():
+        for tensor in self._state_tensors():
             tensor[seq.state_slot].zero_()
         return seq
 

@@ -17,10 +17,13 @@ class PagedKV:
     kv_heads: int
     head_dim: int
     window: int | None = None
+    value_dim: int | None = None      # size of a value if it differs from a key's (None: head_dim)
 
     def __post_init__(self):
-        if self.kv_heads <= 0 or self.head_dim <= 0:
-            raise ValueError("kv_heads and head_dim must be positive")
+        if self.value_dim == self.head_dim:
+            object.__setattr__(self, "value_dim", None)
+        if self.kv_heads <= 0 or self.head_dim <= 0 or (self.value_dim is not None and self.value_dim <= 0):
+            raise ValueError("kv_heads, head_dim and value_dim must be positive")
         if self.window is not None and self.window <= 0:
             raise ValueError("a window must be positive (None means all keys)")
 
@@ -41,8 +44,26 @@ class FixedState:
 
 @dataclass(frozen=True)
 class CacheNeed:
+    """What one cache slot holds: paged keys and values, one fixed-size state, and any number of further
+    fixed-size states by name (a layer whose parts each carry something from token to token: a
+    recurrence, the last inputs of a convolution)."""
     paged: PagedKV | None = None
     state: FixedState | None = None
+    states: tuple = ()                # ((name, FixedState), ...)
+
+    def __post_init__(self):
+        object.__setattr__(self, "states", tuple((str(n), s) for n, s in self.states))
+        names = [n for n, _ in self.states]
+        if len(set(names)) != len(names):
+            raise ValueError("two states of one cache slot share a name")
+
+    def merged(self, other):
+        """This need and OTHER's together (one cache slot for both); at most one of them may page or hold `state`."""
+        if other is None:
+            return self
+        if (self.paged and other.paged) or (self.state and other.state):
+            raise ValueError("two parts of one cache slot both ask for pages, or both for the unnamed state")
+        return CacheNeed(self.paged or other.paged, self.state or other.state, self.states + other.states)
 
 
 @dataclass(frozen=True)
@@ -67,13 +88,15 @@ class CacheLayout:
                 self.slot_group[slot] = (g, i)
         self.state_slots = tuple(slot for slot, need in enumerate(self.needs)
                                  if need is not None and need.state is not None)
+        self.named_state_slots = tuple(slot for slot, need in enumerate(self.needs)
+                                       if need is not None and need.states)
 
     @property
     def shares_prefixes(self):
         """Full pages of a prompt prefix can be reused only if they are all a request holds."""
         return (len(self.groups) == 1 and self.groups[0].spec.window is None
-                and not self.state_slots)
+                and not self.state_slots and not self.named_state_slots)
 
     def bytes_per_token(self, element_bytes):
-        return sum(2 * len(g.slots) * g.spec.kv_heads * g.spec.head_dim * element_bytes
+        return sum(len(g.slots) * g.spec.kv_heads * (g.spec.head_dim + (g.spec.value_dim or g.spec.head_dim)) * element_bytes
                    for g in self.groups)

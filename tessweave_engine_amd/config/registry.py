@@ -2,8 +2,8 @@
 
 The reference has no registry: it whitelists `model_type` and serves both of
 its families with one class (flow_engine/config.py:26, flow_engine/model.py:105).
-Here config.json's `architectures[0]` (or, if absent, its `model_type`) selects
-an entry; the entry's builder assembles a model out of parts.
+Here config.json's `architectures[0]` (or its `architecture`, a single name; or,
+if both are absent, its `model_type`) selects an entry; the entry's builder assembles a model out of parts.
 
 What a configuration class must offer (the engine, the loader and the command
 line read nothing else off it):
@@ -60,7 +60,7 @@ def _load_builtin():
 
 def architecture_for(config_dict) -> Architecture:
     _load_builtin()
-    names = config_dict.get("architectures") or []
+    names = config_dict.get("architectures") or config_dict.get("architecture") or []
     if isinstance(names, str):
         names = [names]
     for name in names:

@@ -1,0 +1,376 @@
+// Attention whose scores are mixed across heads before the softmax, over the paged cache.
+//
+//   keys   [pages][kv_heads][page_size][D]
+//   values [pages][kv_heads][E][page_size]     (transposed inside a page; E may differ from D)
+//
+// For query position i and key position j of one sequence (0 <= i - j < window, or every j <= i
+// without a window):
+//   raw_g(i, j)  = scale * q_ig . k_j,kv(g) - slope_g * (i - j)            (slopes optional)
+//   s_h(i, j)    = sum_g talk[h][g] * raw_g(i, j)                          (talk optional: s = raw)
+//   p_h(i, j)    = exp(s_h(i, j)) / (exp(sink_h) + sum_j' exp(s_h(i, j')))   (sink optional)
+//   out_ih       = out_scale * sum_j p_h(i, j) v_j,kv(h)
+// Scores, the mixing, the softmax and the output sums are float32.
+//
+// Because every head's score at (i, j) needs all heads' raw scores there, a workgroup takes 16
+// query TOKENS with all their heads. Its waves share the heads out between them (HPW heads a
+// wave). Per 16 keys a wave forms S^T = K Q^T for its heads on the matrix unit (accumulator
+// element e of lane (r, g) is query row r against key 4g + e, the same place for every head),
+// leaves the raw scores in LDS, and after one barrier reads all heads' raw scores of its own lane
+// and mixes them for its heads: the mixing needs no exchange between lanes. The probabilities,
+// still in accumulator layout, are the B operand of O^T += V^T P^T. The raw-score buffer exists
+// twice, so one barrier per key tile is enough.
+//
+// Sequences with one token (decode) can have their keys cut into `splits` ranges for separate
+// workgroups; a second kernel merges the partial results in index order.
+#include "tw_common.h"
+
+template <typename T> __device__ __forceinline__ float mx_exp(float v);
+template <> __device__ __forceinline__ float mx_exp<float>(float v) { return expf(v); }
+template <> __device__ __forceinline__ float mx_exp<bf16_t>(float v) { return __expf(v); }
+
+template <typename T> struct MxQuad;
+template <> struct MxQuad<float> { typedef f32x4 Type; };
+template <> struct MxQuad<bf16_t> { typedef bf16x4 Type; };
+
+struct MixedAttnArgs {
+  const void* q; long ldq;           // head h of token n at q + n * ldq + h * D
+  const void* keys; const void* values;
+  const int* block_table; int table_stride;
+  const int* q_start; const int* kv_len;
+  int seq0;
+  void* out; long ldo;               // head h of token n at out + n * ldo + h * E
+  const float* talk;                 // [H][H] or null
+  const float* sink;                 // [H] or null
+  const float* slopes;               // [H] or null
+  float* part;                       // splits > 1: [seq - seq0][split][H][E + 2] (output sums, max, sum)
+  float scale, out_scale;
+  int H, G, D, E, P, window, splits;
+};
+
+// Dynamic LDS: q tile [H][16][D + pad] of T, raw scores [2][H][64] of f32x4, talk [H][H] floats.
+template <typename T>
+__host__ __device__ inline size_t mx_q_row(int D) { return (size_t)D + 16 / sizeof(T); }
+
+template <typename T>
+static size_t mx_lds_bytes(int H, int D) {
+  size_t q = (size_t)H * 16 * mx_q_row<T>(D) * sizeof(T);
+  q = (q + 15) / 16 * 16;
+  return q + (size_t)2 * H * 64 * 16 + (size_t)H * H * 4;
+}
+
+template <typename T, int HPW, int VT>
+__global__ __launch_bounds__(1024) void attn_mixed_kernel(MixedAttnArgs a) {
+  typedef typename Elem<T>::Frag Frag;
+  typedef typename MxQuad<T>::Type Quad;
+  constexpr int EPF = Elem<T>::kPerFrag;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  const int H = a.H, D = a.D, E = a.E, P = a.P;
+  const size_t qrow = mx_q_row<T>(D);
+  T* lds_q = (T*)lds_raw;
+  size_t q_bytes = (size_t)H * 16 * qrow * sizeof(T);
+  q_bytes = (q_bytes + 15) / 16 * 16;
+  f32x4* lds_s = (f32x4*)(lds_raw + q_bytes);
+  float* lds_talk = (float*)(lds_raw + q_bytes + (size_t)2 * H * 64 * 16);
+
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int seq = a.seq0 + blockIdx.y;
+  const int q0 = a.q_start[seq], q_len = a.q_start[seq + 1] - q0;
+  const int tile = blockIdx.x;
+  if (tile * 16 >= q_len) return;
+  const int kv_len = a.kv_len[seq];
+  const int n_rows = min(16, q_len - tile * 16);
+  const int pos0 = kv_len - q_len + tile * 16;              // position of the tile's first row
+  const int t_row = r < n_rows ? pos0 + r : -1;
+  const int* table = a.block_table + (size_t)seq * a.table_stride;
+  const int heads_per_kv = H / a.G;
+  const int chunks = D / EPF, steps = (chunks + 3) / 4, dts = E / 16;
+
+  // ---- stage the tile's queries and the mixing matrix ------------------------------------------------
+  for (int i = threadIdx.x; i < H * 16 * chunks; i += blockDim.x) {
+    const int chunk = i % chunks, row = (i / chunks) % 16, head = i / (chunks * 16);
+    Frag f = Elem<T>::zero();
+    if (row < n_rows)
+      f = tw_load_frag((const T*)a.q + (size_t)(q0 + tile * 16 + row) * a.ldq + (size_t)head * D + chunk * EPF);
+    *reinterpret_cast<Frag*>(lds_q + ((size_t)head * 16 + row) * qrow + chunk * EPF) = f;
+  }
+  for (int i = threadIdx.x; i < H * H; i += blockDim.x)
+    lds_talk[i] = a.talk ? a.talk[i] : ((i / H == i % H) ? 1.f : 0.f);
+  __syncthreads();
+
+  // ---- the key tiles of this workgroup ---------------------------------------------------------------------
+  const int lo = a.window > 0 ? max(0, pos0 - a.window + 1) : 0;       // first key any row of the tile sees
+  const int hi = pos0 + n_rows - 1;                                     // last key (its own position)
+  int tile_lo = lo / 16, tile_hi = hi / 16 + 1;
+  if (a.splits > 1) {
+    const int per = (tile_hi - tile_lo + a.splits - 1) / a.splits;
+    tile_lo = tile_lo + blockIdx.z * per;
+    tile_hi = min(tile_hi, tile_lo + per);
+  }
+  const bool with_sink = a.sink != nullptr && (a.splits == 1 || blockIdx.z == 0);
+
+  float m[HPW], l[HPW];
+  f32x4 acc[HPW][VT];
+  float slope[HPW];
+#pragma unroll
+  for (int i = 0; i < HPW; ++i) {
+    const int head = wave * HPW + i;
+    m[i] = (with_sink && head < H) ? a.sink[head] : -INFINITY;     // the sink: a key of score sink_h and value zero
+    l[i] = (with_sink && head < H) ? 1.f : 0.f;
+    slope[i] = (a.slopes && head < H) ? a.slopes[head] : 0.f;
+#pragma unroll
+    for (int dt = 0; dt < VT; ++dt) acc[i][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  const T* keys = (const T*)a.keys;
+  const T* values = (const T*)a.values;
+  int buf = 0;
+  for (int kt = tile_lo; kt < tile_hi; ++kt, buf ^= 1) {
+    const int p0 = kt * 16;
+    // ---- raw scores of this wave's heads ---------------------------------------------------------------
+    {
+      const int p = p0 + r;
+      int page = -1;
+      if (p < kv_len && p >= lo) page = table[p / P];
+#pragma unroll
+      for (int i = 0; i < HPW; ++i) {
+        const int head = wave * HPW + i;
+        if (head < H) {
+          const int kvh = head / heads_per_kv;
+          const T* k_row = keys + (((size_t)(page < 0 ? 0 : page) * a.G + kvh) * P + p % P) * D;
+          const T* q_row = lds_q + ((size_t)head * 16 + r) * qrow;
+          f32x4 s = {0.f, 0.f, 0.f, 0.f};
+          for (int st = 0; st < steps; ++st) {
+            const int chunk = st * 4 + g;
+            const bool in = chunk < chunks;
+            const Frag kf = (page >= 0 && in) ? tw_load_frag(k_row + chunk * EPF) : Elem<T>::zero();
+            const Frag qf = in ? *reinterpret_cast<const Frag*>(q_row + chunk * EPF) : Elem<T>::zero();
+            tw_mma16(s, kf, qf);
+          }
+#pragma unroll
+          for (int e = 0; e < 4; ++e) s[e] = s[e] * a.scale - slope[i] * (float)(t_row - (p0 + 4 * g + e));
+          lds_s[((size_t)buf * H + head) * 64 + lane] = s;
+        }
+      }
+    }
+    __syncthreads();
+    // ---- mix, mask, online softmax, O^T += V^T P^T ------------------------------------------------------------
+    const int pv = p0 + 4 * g;
+    int vpage = -1;
+    if (pv < kv_len && pv + 3 >= lo) vpage = table[pv / P];
+#pragma unroll
+    for (int i = 0; i < HPW; ++i) {
+      const int head = wave * HPW + i;
+      if (head < H) {
+        f32x4 s = {0.f, 0.f, 0.f, 0.f};
+        for (int other = 0; other < H; ++other) {
+          const float w = lds_talk[head * H + other];
+          const f32x4 raw = lds_s[((size_t)buf * H + other) * 64 + lane];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) s[e] += w * raw[e];
+        }
+        const int lo_row = a.window > 0 ? t_row - a.window + 1 : 0;
+        float mx = -INFINITY;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int p = p0 + 4 * g + e;
+          const bool ok = p < kv_len && p <= t_row && p >= lo_row;
+          s[e] = ok ? s[e] : -INFINITY;
+          mx = fmaxf(mx, s[e]);
+        }
+        mx = tw_rows_max(mx);
+        const float m_new = fmaxf(m[i], mx);
+        const float m_use = m_new == -INFINITY ? 0.f : m_new;
+        const float alpha = mx_exp<T>(m[i] - m_use);
+        f32x4 pr;
+        float sum = 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          pr[e] = mx_exp<T>(s[e] - m_use);
+          sum += pr[e];
+        }
+        sum = tw_rows_sum(sum);
+        l[i] = l[i] * alpha + sum;
+        m[i] = m_new;
+        const int kvh = head / heads_per_kv;
+        const T* v_base = values + ((size_t)(vpage < 0 ? 0 : vpage) * a.G + kvh) * E * P + pv % P;
+#pragma unroll
+        for (int dt = 0; dt < VT; ++dt) {
+          if (dt < dts) {
+            Quad vq;
+            if (vpage >= 0) {
+              vq = *reinterpret_cast<const Quad*>(v_base + (size_t)(dt * 16 + r) * P);
+#pragma unroll
+              for (int e = 0; e < 4; ++e)
+                if (pv + e >= kv_len || pv + e < lo) vq[e] = tw_from_float<T>(0.f);
+            } else {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) vq[e] = tw_from_float<T>(0.f);
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[i][dt][e] *= alpha;
+            tw_mma16_k4(acc[i][dt], vq, pr);
+          }
+        }
+      }
+    }
+  }
+
+  // ---- results: lane (r, g) holds out[row r][16 dt + 4 g + e] ------------------------------------------------------
+#pragma unroll
+  for (int i = 0; i < HPW; ++i) {
+    const int head = wave * HPW + i;
+    if (head >= H || r >= n_rows) continue;
+    if (a.splits == 1) {
+      const float inv = l[i] > 0.f ? a.out_scale / l[i] : 0.f;
+      T* dst = (T*)a.out + (size_t)(q0 + tile * 16 + r) * a.ldo + (size_t)head * E;
+#pragma unroll
+      for (int dt = 0; dt < VT; ++dt)
+        if (dt < dts)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) dst[dt * 16 + 4 * g + e] = tw_from_float<T>(acc[i][dt][e] * inv);
+    } else if (r == 0) {
+      float* dst = a.part + (((size_t)blockIdx.y * a.splits + blockIdx.z) * H + head) * (E + 2);
+#pragma unroll
+      for (int dt = 0; dt < VT; ++dt)
+        if (dt < dts)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) dst[dt * 16 + 4 * g + e] = acc[i][dt][e];
+      if (g == 0) {
+        dst[E] = m[i];
+        dst[E + 1] = l[i];
+      }
+    }
+  }
+}
+
+// Merge the partial results of a one-token sequence's key ranges, in index order. grid (n_seqs, H).
+template <typename T>
+__global__ void attn_mixed_merge_kernel(MixedAttnArgs a) {
+  const int seq = a.seq0 + blockIdx.x, head = blockIdx.y;
+  const int token = a.q_start[seq];
+  const int E = a.E;
+  const float* base = a.part + ((size_t)blockIdx.x * a.splits * a.H + head) * (E + 2);
+  const size_t stride = (size_t)a.H * (E + 2);
+  float m = -INFINITY;
+  for (int s = 0; s < a.splits; ++s) m = fmaxf(m, base[s * stride + E]);
+  const float m_use = m == -INFINITY ? 0.f : m;
+  float l = 0.f;
+  for (int s = 0; s < a.splits; ++s) l += base[s * stride + E + 1] * mx_exp<T>(base[s * stride + E] - m_use);
+  const float inv = l > 0.f ? a.out_scale / l : 0.f;
+  for (int d = threadIdx.x; d < E; d += blockDim.x) {
+    float o = 0.f;
+    for (int s = 0; s < a.splits; ++s) o += base[s * stride + d] * mx_exp<T>(base[s * stride + E] - m_use);
+    ((T*)a.out)[(size_t)token * a.ldo + (size_t)head * E + d] = tw_from_float<T>(o * inv);
+  }
+}
+
+template <typename T, int HPW, int VT>
+static int mixed_launch(const MixedAttnArgs& a, int n_seqs, int tiles, int waves, size_t lds, hipStream_t stream) {
+  auto kernel = attn_mixed_kernel<T, HPW, VT>;
+  if (lds > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return (int)e;
+  }
+  kernel<<<dim3(tiles, n_seqs, a.splits), waves * 64, lds, stream>>>(a);
+  return TW_LAUNCH_RESULT();
+}
+
+template <typename T>
+static int mixed_dispatch(const MixedAttnArgs& a, int n_seqs, int max_q_len, hipStream_t stream) {
+  const int tiles = tw_div_up(max_q_len, 16);
+  // One head a wave up to 16 heads; two a wave (values of up to 64 elements only: the output sums of a
+  // wave's heads live in its registers) up to 32.
+  const int hpw = a.H <= 16 ? 1 : 2;
+  const int waves = tw_div_up(a.H, hpw);
+  const size_t lds = mx_lds_bytes<T>(a.H, a.D);
+  TW_REQUIRE(waves <= 16 && lds <= 150 * 1024 && (hpw == 1 || a.E <= 64));
+  int code;
+  if (hpw == 2)
+    code = mixed_launch<T, 2, 4>(a, n_seqs, tiles, waves, lds, stream);
+  else if (a.E <= 64)
+    code = mixed_launch<T, 1, 4>(a, n_seqs, tiles, waves, lds, stream);
+  else if (a.E <= 128)
+    code = mixed_launch<T, 1, 8>(a, n_seqs, tiles, waves, lds, stream);
+  else
+    code = mixed_launch<T, 1, 16>(a, n_seqs, tiles, waves, lds, stream);
+  if (code != 0 || a.splits == 1) return code;
+  attn_mixed_merge_kernel<T><<<dim3(n_seqs, a.H), 64, 0, stream>>>(a);
+  return TW_LAUNCH_RESULT();
+}
+
+// Key ranges for one-token sequences: enough workgroups to spread over the chip, each with at least 8 key tiles.
+extern "C" int tw_attn_mixed_splits(int n_seqs, int max_kv_len) {
+  if (n_seqs <= 0) return 1;
+  const int tiles = tw_div_up(max_kv_len, 16);
+  int want = 512 / n_seqs;
+  int most = tiles / 8;
+  int s = want < most ? want : most;
+  if (s > 64) s = 64;
+  return s < 1 ? 1 : s;
+}
+
+extern "C" long tw_attn_mixed_workspace_floats(int n_seqs, int q_heads, int value_dim, int splits) {
+  return (long)n_seqs * splits * q_heads * (value_dim + 2);
+}
+
+extern "C" int tw_attn_mixed(int dtype, const void* q, long ldq, const void* keys, const void* values,
+                             const int* block_table, int table_stride, const int* q_start, const int* kv_len,
+                             int seq0, int n_seqs, int max_q_len, void* out, long ldo, const float* talk,
+                             const float* sink, const float* slopes, float* workspace, long workspace_floats,
+                             int q_heads, int kv_heads, int key_dim, int value_dim, int page_size, int window,
+                             float scale, float out_scale, int splits, hipStream_t stream) {
+  TW_REQUIRE(q && keys && values && block_table && q_start && kv_len && out);
+  TW_REQUIRE(n_seqs >= 0 && seq0 >= 0 && max_q_len >= 1 && splits >= 1 && window >= 0);
+  TW_REQUIRE(q_heads >= 1 && q_heads <= 32 && kv_heads >= 1 && q_heads % kv_heads == 0);
+  TW_REQUIRE(key_dim % 16 == 0 && key_dim >= 16 && key_dim <= 256 && value_dim % 16 == 0 && value_dim >= 16 && value_dim <= 256);
+  TW_REQUIRE(page_size > 0 && page_size % 4 == 0);
+  TW_REQUIRE(ldq >= (long)q_heads * key_dim && ldo >= (long)q_heads * value_dim);
+  TW_REQUIRE((uintptr_t)q % 16 == 0 && (uintptr_t)keys % 16 == 0 && (uintptr_t)values % 16 == 0);
+  const int esize = dtype == TW_DTYPE_BF16 ? 2 : 4;
+  TW_REQUIRE((ldq * esize) % 16 == 0);
+  if (splits > 1) {
+    TW_REQUIRE(max_q_len == 1 && workspace != nullptr);
+    TW_REQUIRE(workspace_floats >= tw_attn_mixed_workspace_floats(n_seqs, q_heads, value_dim, splits));
+  }
+  if (n_seqs == 0) return 0;
+  MixedAttnArgs a{q, ldq, keys, values, block_table, table_stride, q_start, kv_len, seq0, out, ldo, talk, sink, slopes,
+                  workspace, scale, out_scale, q_heads, kv_heads, key_dim, value_dim, page_size, window, splits};
+  if (dtype == TW_DTYPE_BF16) return mixed_dispatch<bf16_t>(a, n_seqs, max_q_len, stream);
+  if (dtype == TW_DTYPE_F32) return mixed_dispatch<float>(a, n_seqs, max_q_len, stream);
+  return TW_ERR_BAD_ARGUMENT;
+}
+
+// ---- new keys and values into the pages (no rotation; values transposed inside a page) --------------------------
+template <typename T>
+__global__ void kv_store_kernel(const T* __restrict__ src, long ld, int k_col, int v_col, const int* __restrict__ slots,
+                                T* __restrict__ keys, T* __restrict__ values, int G, int D, int E, int P) {
+  const int n = blockIdx.x;
+  const int slot = slots[n];
+  if (slot < 0) return;
+  const int page = slot / P, at = slot % P;
+  const T* row = src + (size_t)n * ld;
+  for (int i = threadIdx.x; i < G * D; i += blockDim.x) {
+    const int kvh = i / D, d = i % D;
+    keys[(((size_t)page * G + kvh) * P + at) * D + d] = row[k_col + i];
+  }
+  for (int i = threadIdx.x; i < G * E; i += blockDim.x) {
+    const int kvh = i / E, d = i % E;
+    values[(((size_t)page * G + kvh) * E + d) * P + at] = row[v_col + i];
+  }
+}
+
+extern "C" int tw_kv_store(int dtype, const void* src, long ld, int k_col, int v_col, const int* slots, void* keys,
+                           void* values, int n, int kv_heads, int key_dim, int value_dim, int page_size,
+                           hipStream_t stream) {
+  TW_REQUIRE(src && slots && keys && values && n >= 0 && kv_heads > 0 && key_dim > 0 && value_dim > 0 && page_size > 0);
+  TW_REQUIRE(k_col >= 0 && v_col >= 0 && ld >= k_col + (long)kv_heads * key_dim && ld >= v_col + (long)kv_heads * value_dim);
+  if (n == 0) return 0;
+  if (dtype == TW_DTYPE_BF16)
+    kv_store_kernel<bf16_t><<<n, 128, 0, stream>>>((const bf16_t*)src, ld, k_col, v_col, slots, (bf16_t*)keys, (bf16_t*)values,
+                                                    kv_heads, key_dim, value_dim, page_size);
+  else if (dtype == TW_DTYPE_F32)
+    kv_store_kernel<float><<<n, 128, 0, stream>>>((const float*)src, ld, k_col, v_col, slots, (float*)keys, (float*)values,
+                                                  kv_heads, key_dim, value_dim, page_size);
+  else return TW_ERR_BAD_ARGUMENT;
+  return TW_LAUNCH_RESULT();
+}

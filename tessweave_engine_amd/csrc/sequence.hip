@@ -1,0 +1,332 @@
+// Kernels over a step's flat ragged batch that look back along a sequence or carry per-request state:
+// a learned position table added to the embedding, a short causal convolution over time with its last
+// inputs kept per request (optionally behind an RMS norm), a gated linear recurrence, the per-layer token
+// input, and the weighted sum over the results of all earlier layers.
+//
+// The batch is n_tokens rows grouped by sequence: sequence s owns rows q_start[s] .. q_start[s+1]-1 at
+// positions kv_len[s] - q_len .. kv_len[s] - 1. State lives in float32 arrays indexed by the request's
+// state slot. Everything here is float32 arithmetic; only inputs that come from a projection and outputs
+// that feed one have the compute type.
+#include "tw_common.h"
+
+__device__ __forceinline__ float tw_gelu_tanh(float z) {
+  return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+__device__ __forceinline__ float tw_sigmoid(float z) { return 1.f / (1.f + expf(-z)); }
+
+// The sequence that owns token row `row` (q_start is ascending, q_start[n_seqs] = n_tokens).
+__device__ __forceinline__ int tw_seq_of_row(const int* __restrict__ q_start, int n_seqs, int row) {
+  int lo = 0, hi = n_seqs - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (q_start[mid] <= row) lo = mid; else hi = mid - 1;
+  }
+  return lo;
+}
+
+// ---- x[n] += table[ids[n]]; optionally keep a copy of the sum -------------------------------------------
+template <typename T>
+__global__ void add_table_rows_kernel(float* __restrict__ x, const T* __restrict__ table, const int* __restrict__ ids,
+                                      int width, int rows, float* __restrict__ copy) {
+  const int n = blockIdx.x;
+  int id = ids[n];
+  id = id < 0 ? 0 : (id >= rows ? rows - 1 : id);
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    const float v = x[(size_t)n * width + c] + tw_to_float(table[(size_t)id * width + c]);
+    x[(size_t)n * width + c] = v;
+    if (copy) copy[(size_t)n * width + c] = v;
+  }
+}
+
+extern "C" int tw_add_table_rows(int dtype, float* x, const void* table, const int* ids, int n, int width, int rows,
+                                 float* copy, hipStream_t stream) {
+  TW_REQUIRE(x && table && ids && n >= 0 && width > 0 && rows > 0);
+  if (n == 0) return 0;
+  if (dtype == TW_DTYPE_BF16)
+    add_table_rows_kernel<bf16_t><<<n, 256, 0, stream>>>(x, (const bf16_t*)table, ids, width, rows, copy);
+  else if (dtype == TW_DTYPE_F32)
+    add_table_rows_kernel<float><<<n, 256, 0, stream>>>(x, (const float*)table, ids, width, rows, copy);
+  else
+    return TW_ERR_BAD_ARGUMENT;
+  return TW_LAUNCH_RESULT();
+}
+
+// ---- short causal convolution over time, with state ------------------------------------------------------
+// v_t = NORM ? src_t * rsqrt(mean(src_t^2) + eps) * norm_w : src_t          (per channel c)
+// out_t = identity * v_t + sum_j taps[c][j] * v_(t - K + 1 + j) + bias[c]
+// Rows before this step's first token of the sequence come from the request's state, rows before the
+// sequence's start are zeros. The state holds the last K - 1 values v in order (entry k is position
+// len - (K - 1) + k) and exists twice: a step reads copy `phase` and the block of a sequence's last token
+// writes copy `1 - phase`, so no block ever reads what another block of the same launch writes.
+#define TW_CONV_MAX_TAPS 8
+
+struct ConvArgs {
+  const void* src; long ld_src;       // [n][ld_src], channel c at column c
+  const float* norm_w;                // NORM only
+  const float* taps;                  // [C][K]
+  const float* bias;                  // [C] or null
+  float* state;                       // [requests][2][K - 1][C]
+  const int* q_start; const int* kv_len; const int* state_slots; const int* phase;
+  void* out; long ld_out;             // compute type, or null
+  float* out32; long ld_out32;        // float32, or null
+  int n_seqs, C, K;
+  float eps, identity;
+};
+
+template <typename SrcT, typename OutT, bool NORM>
+__global__ __launch_bounds__(256) void causal_conv_kernel(ConvArgs a) {
+  __shared__ float red[16];
+  __shared__ float rinv[TW_CONV_MAX_TAPS];
+  const int row = blockIdx.x;
+  const int s = tw_seq_of_row(a.q_start, a.n_seqs, row);
+  const int first = a.q_start[s], q_len = a.q_start[s + 1] - first;
+  const int len = a.kv_len[s];
+  const int start = len - q_len;                 // position of the step's first token of this sequence
+  const int pos = start + (row - first);
+  const int K = a.K, C = a.C;
+  const int slot = a.state_slots[s], ph = a.phase[s] & 1;
+  const float* old_state = a.state + ((size_t)slot * 2 + ph) * (size_t)(K - 1) * C;
+  float* new_state = a.state + ((size_t)slot * 2 + (1 - ph)) * (size_t)(K - 1) * C;
+  const bool last = pos == len - 1;
+  const SrcT* src = (const SrcT*)a.src;
+
+  if (NORM) {
+    for (int j = 0; j < K; ++j) {
+      const int p = pos - (K - 1) + j;
+      float sum = 0.f;
+      if (p >= start) {
+        const SrcT* r = src + (size_t)(first + p - start) * a.ld_src;
+        for (int c = threadIdx.x; c < C; c += blockDim.x) {
+          const float v = tw_to_float(r[c]);
+          sum += v * v;
+        }
+      }
+      sum = tw_block_sum(sum, red);
+      if (threadIdx.x == 0) rinv[j] = rsqrtf(sum / (float)C + a.eps);
+    }
+    __syncthreads();
+  }
+  for (int c = threadIdx.x; c < C; c += blockDim.x) {
+    float acc = a.bias ? a.bias[c] : 0.f;
+    const float nw = NORM ? a.norm_w[c] : 1.f;
+    for (int j = 0; j < K; ++j) {
+      const int p = pos - (K - 1) + j;
+      float v = 0.f;
+      if (p >= start) {
+        v = tw_to_float(src[(size_t)(first + p - start) * a.ld_src + c]);
+        if (NORM) v = v * rinv[j] * nw;
+      } else if (p >= 0) {
+        v = old_state[(size_t)(p - start + K - 1) * C + c];
+      }
+      acc += a.taps[(size_t)c * K + j] * v;
+      if (j == K - 1) acc += a.identity * v;
+      if (last && j >= 1) new_state[(size_t)(j - 1) * C + c] = v;
+    }
+    if (a.out) ((OutT*)a.out)[(size_t)row * a.ld_out + c] = tw_from_float<OutT>(acc);
+    if (a.out32) a.out32[(size_t)row * a.ld_out32 + c] = acc;
+  }
+}
+
+// src_kind: 0 float32 rows, 1 rows of the compute type. norm_w non-null: RMS norm of the source rows first
+// (float32 rows only).
+extern "C" int tw_causal_conv(int dtype, int src_f32, const void* src, long ld_src, const float* norm_w, float eps,
+                              const float* taps, const float* bias, float identity, float* state,
+                              const int* q_start, const int* kv_len, const int* state_slots, const int* phase,
+                              void* out, long ld_out, float* out32, long ld_out32, int n_tokens, int n_seqs,
+                              int C, int K, hipStream_t stream) {
+  TW_REQUIRE(src && taps && state && q_start && kv_len && state_slots && phase && (out || out32));
+  TW_REQUIRE(n_tokens >= 0 && n_seqs >= 1 && C > 0 && K >= 1 && K <= TW_CONV_MAX_TAPS);
+  TW_REQUIRE(ld_src >= C && (!out || ld_out >= C) && (!out32 || ld_out32 >= C));
+  TW_REQUIRE(!norm_w || src_f32);
+  if (n_tokens == 0) return 0;
+  ConvArgs a{src, ld_src, norm_w, taps, bias, state, q_start, kv_len, state_slots, phase,
+             out, ld_out, out32, ld_out32, n_seqs, C, K, eps, identity};
+  const bool bf = dtype == TW_DTYPE_BF16;
+  TW_REQUIRE(bf || dtype == TW_DTYPE_F32);
+  if (norm_w) {
+    if (bf) causal_conv_kernel<float, bf16_t, true><<<n_tokens, 256, 0, stream>>>(a);
+    else causal_conv_kernel<float, float, true><<<n_tokens, 256, 0, stream>>>(a);
+  } else if (src_f32) {
+    if (bf) causal_conv_kernel<float, bf16_t, false><<<n_tokens, 256, 0, stream>>>(a);
+    else causal_conv_kernel<float, float, false><<<n_tokens, 256, 0, stream>>>(a);
+  } else {
+    if (bf) causal_conv_kernel<bf16_t, bf16_t, false><<<n_tokens, 256, 0, stream>>>(a);
+    else causal_conv_kernel<float, float, false><<<n_tokens, 256, 0, stream>>>(a);
+  }
+  return TW_LAUNCH_RESULT();
+}
+
+// ---- gated linear recurrence ---------------------------------------------------------------------------------
+// Per sequence and channel, over the step's tokens in order:
+//   r = sigmoid(gates[t][ga(c)]), i = sigmoid(gates[t][gi(c)])
+//   a = exp(-decay * r * softplus(lam[c]))
+//   S = a * S + sqrt(1 - a^2) * i * u[t][c]                 (S float32, kept per request)
+//   out[t][c] = out_scale * S * gelu_tanh(branch[t][c])
+// The gates of block b (bs = C / blocks channels) lie at columns [2 b bs, 2 b bs + bs) (recurrence gate)
+// and [2 b bs + bs, 2 (b + 1) bs) (input gate): one packed product per block wrote them.
+struct RecurrenceArgs {
+  const float* gates; long ld_gates;
+  const float* u; long ld_u;
+  const void* branch; long ld_branch;
+  const float* lam;
+  float* state;                       // [requests][C]
+  const int* q_start; const int* state_slots;
+  void* out; long ld_out;
+  int C, block_size;
+  float decay, out_scale;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void gated_recurrence_kernel(RecurrenceArgs a) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= a.C) return;
+  const int s = blockIdx.y;
+  const int first = a.q_start[s], end = a.q_start[s + 1];
+  float* st = a.state + (size_t)a.state_slots[s] * a.C + c;
+  float S = *st;
+  const float lam = a.lam[c];
+  const float unit = a.decay * (lam > 20.f ? lam : log1pf(expf(lam)));
+  const int b = c / a.block_size, k = c % a.block_size;
+  const int ga = 2 * b * a.block_size + k, gi = ga + a.block_size;
+  const T* branch = (const T*)a.branch;
+  T* out = (T*)a.out;
+  for (int t = first; t < end; ++t) {
+    const float r = tw_sigmoid(a.gates[(size_t)t * a.ld_gates + ga]);
+    const float i = tw_sigmoid(a.gates[(size_t)t * a.ld_gates + gi]);
+    const float la = -unit * r;
+    const float dec = expf(la);
+    const float norm = sqrtf(fmaxf(0.f, -expm1f(2.f * la)));          // sqrt(1 - a^2) without cancellation
+    S = dec * S + norm * i * a.u[(size_t)t * a.ld_u + c];
+    const float y = tw_gelu_tanh(tw_to_float(branch[(size_t)t * a.ld_branch + c]));
+    out[(size_t)t * a.ld_out + c] = tw_from_float<T>(a.out_scale * S * y);
+  }
+  *st = S;
+}
+
+extern "C" int tw_gated_recurrence(int dtype, const float* gates, long ld_gates, const float* u, long ld_u,
+                                   const void* branch, long ld_branch, const float* lam, float* state,
+                                   const int* q_start, const int* state_slots, void* out, long ld_out, int n_seqs,
+                                   int C, int blocks, float decay, float out_scale, hipStream_t stream) {
+  TW_REQUIRE(gates && u && branch && lam && state && q_start && state_slots && out);
+  TW_REQUIRE(n_seqs >= 0 && C > 0 && blocks > 0 && C % blocks == 0);
+  TW_REQUIRE(ld_gates >= 2 * C && ld_u >= C && ld_branch >= C && ld_out >= C);
+  if (n_seqs == 0) return 0;
+  RecurrenceArgs a{gates, ld_gates, u, ld_u, branch, ld_branch, lam, state, q_start, state_slots, out, ld_out,
+                   C, C / blocks, decay, out_scale};
+  dim3 grid(tw_div_up(C, 256), n_seqs);
+  if (dtype == TW_DTYPE_BF16) gated_recurrence_kernel<bf16_t><<<grid, 256, 0, stream>>>(a);
+  else if (dtype == TW_DTYPE_F32) gated_recurrence_kernel<float><<<grid, 256, 0, stream>>>(a);
+  else return TW_ERR_BAD_ARGUMENT;
+  return TW_LAUNCH_RESULT();
+}
+
+// ---- out = scale * act(gate) * up for [n][2F] rows holding gate | up -------------------------------------------
+template <typename T>
+__global__ void gelu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, long n, int inter, float scale) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n * inter) return;
+  const long row = i / inter;
+  const int col = (int)(i % inter);
+  const float g = tw_to_float(gu[row * 2 * inter + col]), u = tw_to_float(gu[row * 2 * inter + inter + col]);
+  out[i] = tw_from_float<T>(scale * tw_gelu_tanh(g) * u);
+}
+
+extern "C" int tw_gelu_mul(int dtype, const void* gu, void* out, int n, int inter, float scale, hipStream_t stream) {
+  TW_REQUIRE(gu && out && n >= 0 && inter > 0);
+  if (n == 0) return 0;
+  const long total = (long)n * inter;
+  const int blocks = tw_div_up(total, 256);
+  if (dtype == TW_DTYPE_BF16) gelu_mul_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, n, inter, scale);
+  else if (dtype == TW_DTYPE_F32) gelu_mul_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gu, (float*)out, n, inter, scale);
+  else return TW_ERR_BAD_ARGUMENT;
+  return TW_LAUNCH_RESULT();
+}
+
+// ---- float32 rows rounded to the compute type ------------------------------------------------------------------
+template <typename T>
+__global__ void round_rows_kernel(const float* __restrict__ x, T* __restrict__ out, long total) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < total) out[i] = tw_from_float<T>(x[i]);
+}
+
+extern "C" int tw_round_rows(int dtype, const float* x, void* out, long total, hipStream_t stream) {
+  TW_REQUIRE(x && out && total >= 0);
+  if (total == 0) return 0;
+  const int blocks = tw_div_up(total, 256);
+  if (dtype == TW_DTYPE_BF16) round_rows_kernel<bf16_t><<<blocks, 256, 0, stream>>>(x, (bf16_t*)out, total);
+  else if (dtype == TW_DTYPE_F32) round_rows_kernel<float><<<blocks, 256, 0, stream>>>(x, (float*)out, total);
+  else return TW_ERR_BAD_ARGUMENT;
+  return TW_LAUNCH_RESULT();
+}
+
+// ---- the per-layer token input's gate: out[n][k] = gelu_tanh(pre[n][k]) * table[token n][offset + k] ------------
+template <typename T>
+__global__ void token_gate_kernel(const float* __restrict__ pre, const T* __restrict__ table, long ld_table,
+                                  const int* __restrict__ ids, const int* __restrict__ feed, int n_feed, int vocab,
+                                  int offset, T* __restrict__ out, int n, int dim) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (long)n * dim) return;
+  const int row = (int)(i / dim), k = (int)(i % dim);
+  int id = ids[row];
+  if (id < 0) id = (feed && -1 - id < n_feed) ? feed[-1 - id] : 0;
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+  out[i] = tw_from_float<T>(tw_gelu_tanh(pre[i]) * tw_to_float(table[(size_t)id * ld_table + offset + k]));
+}
+
+extern "C" int tw_token_gate(int dtype, const float* pre, const void* table, long ld_table, const int* ids,
+                             const int* feed, int n_feed, int vocab, int offset, void* out, int n, int dim,
+                             hipStream_t stream) {
+  TW_REQUIRE(pre && table && ids && out && n >= 0 && dim > 0 && offset >= 0 && offset + dim <= ld_table && vocab > 0);
+  if (n == 0) return 0;
+  const int blocks = tw_div_up((long)n * dim, 256);
+  if (dtype == TW_DTYPE_BF16)
+    token_gate_kernel<bf16_t><<<blocks, 256, 0, stream>>>(pre, (const bf16_t*)table, ld_table, ids, feed, n_feed, vocab, offset, (bf16_t*)out, n, dim);
+  else if (dtype == TW_DTYPE_F32)
+    token_gate_kernel<float><<<blocks, 256, 0, stream>>>(pre, (const float*)table, ld_table, ids, feed, n_feed, vocab, offset, (float*)out, n, dim);
+  else return TW_ERR_BAD_ARGUMENT;
+  return TW_LAUNCH_RESULT();
+}
+
+// ---- end of a layer: add a unit-norm branch, keep the layer's result, mix the results so far --------------------
+//   if y:  x[n] += mult * y[n] * rsqrt(mean(y[n]^2) + eps) * w
+//   history[layer + 1][n] = x[n]
+//   if mix: x[n] = sum_{j <= layer + 1} mix[j] * history[j][n]
+// history[j] lies at history + j * history_stride.
+__global__ __launch_bounds__(256) void layer_end_kernel(float* __restrict__ x, const float* __restrict__ y,
+                                                        const float* __restrict__ w, float eps, float mult,
+                                                        float* __restrict__ history, long history_stride, int layer,
+                                                        const float* __restrict__ mix, int width) {
+  __shared__ float red[16];
+  const size_t row = (size_t)blockIdx.x * width;
+  float scale = 0.f;
+  if (y) {
+    float sum = 0.f;
+    for (int c = threadIdx.x; c < width; c += blockDim.x) {
+      const float v = y[row + c];
+      sum += v * v;
+    }
+    sum = tw_block_sum(sum, red);
+    scale = mult * rsqrtf(sum / (float)width + eps);
+  }
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    float v = x[row + c];
+    if (y) v += scale * y[row + c] * w[c];
+    if (history) history[(size_t)(layer + 1) * history_stride + row + c] = v;
+    if (mix) {
+      float acc = mix[layer + 1] * v;
+      for (int j = 0; j <= layer; ++j) acc += mix[j] * history[(size_t)j * history_stride + row + c];
+      v = acc;
+    }
+    x[row + c] = v;
+  }
+}
+
+extern "C" int tw_layer_end(float* x, const float* y, const float* w, float eps, float mult, float* history,
+                            long history_stride, int layer, const float* mix, int n, int width, hipStream_t stream) {
+  TW_REQUIRE(x && n >= 0 && width > 0 && layer >= 0 && (!y || w) && (!mix || history));
+  TW_REQUIRE(!history || history_stride >= (long)n * width);
+  if (n == 0) return 0;
+  layer_end_kernel<<<n, 256, 0, stream>>>(x, y, w, eps, mult, history, history_stride, layer, mix, width);
+  return TW_LAUNCH_RESULT();
+}

@@ -23,7 +23,7 @@ from pathlib import Path
 import sys
 
 PAGE_SIZE = 16
-MAX_LIVE_REQUESTS = 64
+MAX_LIVE_REQUESTS = 4
 
 
 def parse_args(argv=None):
@@ -35,6 +35,8 @@ def parse_args(argv=None):
                    help="most tokens live requests hold at once (each rounded up to a multiple of 64)")
     p.add_argument("--page-size", type=int, default=PAGE_SIZE,
                    help="tokens per cache page: any size the engine takes (a multiple of 4)")
+    p.add_argument("--max-requests", type=int, default=MAX_LIVE_REQUESTS,
+                   help="requests that can be live at once: the state slots the cache is made with")
     p.add_argument("--no-graphs", action="store_true", help="never replay decode steps from HIP graphs")
     return p.parse_args(argv)
 
@@ -63,7 +65,9 @@ def run(args, lines, out=sys.stdout):
     out_dir.mkdir(parents=True, exist_ok=True)
     model = load_model(args.model, dtype=args.dtype, device="cuda:0")
     pages = pool_pages(args.max_tokens, args.page_size)
-    cache = CacheManager(model.cache_layout(), args.page_size, pages, MAX_LIVE_REQUESTS, dtype=args.dtype,
+    if args.max_requests <= 0:
+        raise SystemExit("--max-requests must be positive")
+    cache = CacheManager(model.cache_layout(), args.page_size, pages, args.max_requests, dtype=args.dtype,
                          device=model.device, prefix_cache=False,
                          max_request_tokens=pages * args.page_size)
     stepper = Stepper(model, cache, max_step_tokens=256, use_graphs=not args.no_graphs)

@@ -108,6 +108,7 @@ class Stepper:
         add("q_start", max_seqs + 1)
         add("kv_len", max_seqs)
         add("state_slots", max_seqs)
+        add("state_phase", max_seqs)
         add("logit_rows", max_tokens)
         for g in range(n_groups):
             add(f"slots{g}", max_tokens)
@@ -193,6 +194,7 @@ class Stepper:
         """Record in the cache that the step's tokens are now held."""
         for e in ordered:
             self.cache.advance(e.seq, e.seq.computed + len(e.tokens))
+            e.seq.steps += 1
         self.steps += 1
 
     def upload(self, ctx):
@@ -281,6 +283,7 @@ class Stepper:
         put("q_start", q_start)
         put("kv_len", kv_len)
         put("state_slots", slots_of)
+        put("state_phase", np.fromiter((e.seq.steps & 1 for e in ordered), dtype=np.int64, count=n_seqs))
         put("logit_rows", np.asarray(rows, dtype=np.int64))
         page = self.cache.page_size
         width = self.cache.table_width
@@ -304,6 +307,7 @@ class Stepper:
         ctx.q_start = self._dev("q_start", n_seqs + 1)
         ctx.kv_len = self._dev("kv_len", n_seqs)
         ctx.state_slots = self._dev("state_slots", n_seqs)
+        ctx.state_phase = self._dev("state_phase", n_seqs)
         ctx.logit_rows = self._dev("logit_rows", n_logits)
         ctx.groups = [GroupStep(self._dev(f"table{g}", n_seqs * width).view(n_seqs, width),
                                 self._dev(f"slots{g}", n_tokens)) for g in range(len(self.cache.pools))]

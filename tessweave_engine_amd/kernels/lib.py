@@ -36,6 +36,17 @@ _SIGNATURES = {
     "tw_attn_prefill_split": (I, [I, I, I, I, I, I, ctypes.POINTER(c_int), ctypes.POINTER(c_int)]),
     "tw_attn_prefill_workspace_floats": (L, [I, I, I, I]),
     "tw_attn_prefill": (I, [I, P, L, P, P, P, I, P, P, I, I, I, P, L, P, L, I, I, I, I, I, I, I, I, I, F, F, I, P]),
+    "tw_add_table_rows": (I, [I, P, P, P, I, I, I, P, P]),
+    "tw_causal_conv": (I, [I, I, P, L, P, F, P, P, F, P, P, P, P, P, P, L, P, L, I, I, I, I, P]),
+    "tw_gated_recurrence": (I, [I, P, L, P, L, P, L, P, P, P, P, P, L, I, I, I, F, F, P]),
+    "tw_gelu_mul": (I, [I, P, P, I, I, F, P]),
+    "tw_round_rows": (I, [I, P, P, L, P]),
+    "tw_token_gate": (I, [I, P, P, L, P, P, I, I, I, P, I, I, P]),
+    "tw_layer_end": (I, [P, P, P, F, F, P, L, I, P, I, I, P]),
+    "tw_attn_mixed_splits": (I, [I, I]),
+    "tw_attn_mixed_workspace_floats": (L, [I, I, I, I]),
+    "tw_attn_mixed": (I, [I, P, L, P, P, P, I, P, P, I, I, I, P, L, P, P, P, P, L, I, I, I, I, I, I, F, F, I, P]),
+    "tw_kv_store": (I, [I, P, L, I, I, P, P, P, I, I, I, I, I, P]),
     "tw_sampling_uniform": (F, [c_uint64, c_uint64]),
     "tw_sample_workspace_bytes": (L, [I]),
     "tw_sample_rows": (I, [P, L, I, I, P, P, P, P, P, L, P]),

@@ -454,3 +454,203 @@ def sample_rows(logits, out, temperature=None, seeds=None, counters=None, worksp
                                    _dev(out, torch.int32, "out"), _dev(workspace),
                                    workspace.numel() * workspace.element_size(), _stream()), "sample_rows")
     return out
+
+
+# ---- kernels over sequences: position table, causal convolution with state, gated recurrence, layer end ---------
+
+def add_table_rows(x, table, ids, copy=None):
+    """x[n] += table[ids[n]] (x float32 [n, width]); COPY, if given, receives the sums as well."""
+    n, width = x.shape
+    _need(x.is_contiguous() and table.dim() == 2 and table.is_contiguous() and table.shape[1] == width,
+          "add_table_rows: x [n, width] and table [rows, width] must be contiguous")
+    _need(ids.numel() == n, "one row id per token is needed")
+    if copy is not None:
+        _need(copy.is_contiguous() and tuple(copy.shape) == (n, width), "the copy must have x's shape")
+    check(library().tw_add_table_rows(dtype_id(table.dtype), _dev(x, torch.float32, "x"), _dev(table),
+                                      _dev(ids, torch.int32, "ids"), n, width, table.shape[0],
+                                      _dev(copy, torch.float32, "copy") if copy is not None else None, _stream()),
+          "add_table_rows")
+    return x
+
+
+CONV_MAX_TAPS = 8
+
+
+def causal_conv(src, taps, state, q_start, kv_len, state_slots, phase, n_seqs, out=None, out32=None, norm_weight=None,
+                eps=0.0, bias=None, identity=0.0):
+    """Causal convolution over time on each channel, with the request's last inputs as state.
+
+    v_t = src_t (or its RMS norm times norm_weight, for float32 rows); out_t = identity * v_t +
+    sum_j taps[:, j] * v_(t - K + 1 + j) + bias. state float32 [requests, 2, max(K - 1, 1), C]: copy
+    phase[s] is read, the other copy written. out has the compute type, out32 is float32; either may be None.
+    """
+    n, C, ld_src = _rows(src, "src")
+    K = taps.shape[1]
+    _need(taps.dtype == torch.float32 and taps.is_contiguous() and taps.shape[0] == C, "taps must be float32 [C, K]")
+    _need(1 <= K <= CONV_MAX_TAPS, f"a convolution has 1 to {CONV_MAX_TAPS} taps")
+    _need(state.dtype == torch.float32 and state.is_contiguous() and state.dim() == 4
+          and tuple(state.shape[1:]) == (2, max(K - 1, 1), C), "state must be float32 [requests, 2, max(K - 1, 1), C]")
+    _need(out is not None or out32 is not None, "causal_conv needs an output")
+    ld_out = ld_out32 = 0
+    compute = src.dtype
+    if out is not None:
+        no, co, ld_out = _rows(out, "out")
+        _need((no, co) == (n, C), "out has the wrong shape")
+        compute = out.dtype
+    if out32 is not None:
+        no, co, ld_out32 = _rows(out32, "out32")
+        _need((no, co) == (n, C) and out32.dtype == torch.float32, "out32 must be float32 [n, C]")
+    src_f32 = src.dtype == torch.float32
+    _need(src_f32 or src.dtype == compute, "src must be float32 or of the output's type")
+    if norm_weight is not None:
+        _need(src_f32 and norm_weight.numel() == C, "a norm needs float32 rows and a weight per channel")
+    if bias is not None:
+        _need(bias.numel() == C and bias.dtype == torch.float32, "bias must be float32 [C]")
+    _need(q_start.numel() >= n_seqs + 1 and kv_len.numel() >= n_seqs and state_slots.numel() >= n_seqs
+          and phase.numel() >= n_seqs, "sequence metadata is too short")
+    check(library().tw_causal_conv(dtype_id(compute), 1 if src_f32 else 0, _dev(src), ld_src,
+                                   _dev(norm_weight, torch.float32, "norm_weight") if norm_weight is not None else None,
+                                   float(eps), _dev(taps), _dev(bias) if bias is not None else None, float(identity),
+                                   _dev(state), _dev(q_start, torch.int32, "q_start"), _dev(kv_len, torch.int32, "kv_len"),
+                                   _dev(state_slots, torch.int32, "state_slots"), _dev(phase, torch.int32, "phase"),
+                                   _dev(out) if out is not None else None, ld_out,
+                                   _dev(out32) if out32 is not None else None, ld_out32, n, int(n_seqs), C, K, _stream()),
+          "causal_conv")
+
+
+def gated_recurrence(gates, u, branch, lam, state, q_start, state_slots, n_seqs, out, blocks, decay, out_scale=1.0):
+    """The gated linear recurrence S = a S + sqrt(1 - a^2) i u per sequence and channel, a = exp(-decay *
+    sigmoid(gate_a) * softplus(lam)); out = out_scale * S * gelu_tanh(branch). gates float32 [n, 2C], block b's
+    recurrence gates at columns [2 b C/blocks, ...) followed by its input gates; u float32 [n, C]; branch and
+    out have the compute type; state float32 [requests, C]."""
+    n, C, ld_u = _rows(u, "u")
+    ng, cg, ld_g = _rows(gates, "gates")
+    nb, cb, ld_b = _rows(branch, "branch")
+    no, co, ld_o = _rows(out, "out")
+    _need(gates.dtype == torch.float32 and u.dtype == torch.float32, "gates and u must be float32")
+    _need((ng, cg) == (n, 2 * C) and (nb, cb) == (n, C) and (no, co) == (n, C) and branch.dtype == out.dtype,
+          "gated_recurrence shapes do not agree")
+    _need(C % blocks == 0 and lam.numel() == C and lam.dtype == torch.float32, "lam must be float32 [C], C a multiple of blocks")
+    _need(state.dtype == torch.float32 and state.is_contiguous() and state.shape[-1] == C and state.dim() == 2,
+          "state must be float32 [requests, C]")
+    check(library().tw_gated_recurrence(dtype_id(out.dtype), _dev(gates), ld_g, _dev(u), ld_u, _dev(branch), ld_b,
+                                        _dev(lam), _dev(state), _dev(q_start, torch.int32, "q_start"),
+                                        _dev(state_slots, torch.int32, "state_slots"), _dev(out), ld_o, int(n_seqs), C,
+                                        int(blocks), float(decay), float(out_scale), _stream()), "gated_recurrence")
+    return out
+
+
+def gelu_mul(gate_up, out, scale=1.0):
+    """out[n, i] = scale * gelu_tanh(gate_up[n, i]) * gate_up[n, inter + i]."""
+    _need(gate_up.dim() == 2 and gate_up.is_contiguous() and gate_up.shape[1] % 2 == 0, "gate_up must be contiguous [n, 2*inter]")
+    n, inter = gate_up.shape[0], gate_up.shape[1] // 2
+    _need(out.is_contiguous() and tuple(out.shape) == (n, inter) and out.dtype == gate_up.dtype,
+          "gelu_mul output has the wrong shape or type")
+    check(library().tw_gelu_mul(dtype_id(gate_up.dtype), _dev(gate_up), _dev(out), n, inter, float(scale), _stream()), "gelu_mul")
+    return out
+
+
+def round_rows(x, out):
+    """out = x rounded to out's type (x float32, both contiguous and of one shape)."""
+    _need(x.is_contiguous() and out.is_contiguous() and x.shape == out.shape, "round_rows operands must be contiguous and alike")
+    check(library().tw_round_rows(dtype_id(out.dtype), _dev(x, torch.float32, "x"), _dev(out), x.numel(), _stream()), "round_rows")
+    return out
+
+
+def token_gate(pre, table, ids, offset, out, feed=None):
+    """out[n, k] = gelu_tanh(pre[n, k]) * table[ids[n], offset + k]; an id -1 - k stands for feed[k]."""
+    n, dim = pre.shape
+    _need(pre.dtype == torch.float32 and pre.is_contiguous() and out.is_contiguous() and tuple(out.shape) == (n, dim),
+          "token_gate: pre float32 [n, dim] and out [n, dim] must be contiguous")
+    _need(table.dim() == 2 and table.is_contiguous() and table.dtype == out.dtype and offset + dim <= table.shape[1],
+          "token_gate: the table must be contiguous, of out's type, and hold the asked columns")
+    check(library().tw_token_gate(dtype_id(out.dtype), _dev(pre), _dev(table), table.shape[1], _dev(ids, torch.int32, "ids"),
+                                  _dev(feed, torch.int32, "feed") if feed is not None else None,
+                                  feed.numel() if feed is not None else 0, table.shape[0], int(offset), _dev(out), n, dim,
+                                  _stream()), "token_gate")
+    return out
+
+
+def layer_end(x, layer, branch=None, branch_weight=None, eps=0.0, mult=1.0, history=None, mix=None):
+    """x += mult * branch / rms(branch) * branch_weight (if a branch is given); history[layer + 1] = x;
+    then, with MIX (float32 [layer + 2]), x = sum_j mix[j] * history[j]. history float32 [layers + 1, rows, width]
+    (rows >= n: a buffer sized for the largest step)."""
+    n, width = x.shape
+    _need(x.dtype == torch.float32 and x.is_contiguous(), "x must be contiguous float32 [n, width]")
+    if branch is not None:
+        _need(branch.dtype == torch.float32 and branch.is_contiguous() and tuple(branch.shape) == (n, width)
+              and branch_weight is not None and branch_weight.numel() == width, "the branch must be float32 [n, width] with a weight")
+    stride = 0
+    if history is not None:
+        _need(history.dtype == torch.float32 and history.is_contiguous() and history.dim() == 3
+              and history.shape[2] == width and history.shape[1] >= n and history.shape[0] >= layer + 2,
+              "history must be float32 [layers + 1, rows >= n, width]")
+        stride = history.shape[1] * width
+    if mix is not None:
+        _need(history is not None and mix.dtype == torch.float32 and mix.numel() == layer + 2, "mix must be float32 [layer + 2]")
+    check(library().tw_layer_end(_dev(x), _dev(branch) if branch is not None else None,
+                                 _dev(branch_weight, torch.float32, "branch_weight") if branch is not None else None,
+                                 float(eps), float(mult), _dev(history) if history is not None else None, stride, int(layer),
+                                 _dev(mix) if mix is not None else None, n, width, _stream()), "layer_end")
+    return x
+
+
+# ---- attention with scores mixed across heads ------------------------------------------------------------------------
+
+def attn_mixed_splits(n_seqs, max_kv_len):
+    return int(library().tw_attn_mixed_splits(int(n_seqs), int(max_kv_len)))
+
+
+def attn_mixed_workspace_floats(n_seqs, q_heads, value_dim, splits):
+    return int(library().tw_attn_mixed_workspace_floats(int(n_seqs), q_heads, value_dim, int(splits)))
+
+
+def kv_store(src, k_col, v_col, slots, keys, values, kv_heads, key_dim, value_dim):
+    """Row n's keys src[n, k_col : k_col + kv_heads * key_dim] and values src[n, v_col : ...] into the page slot
+    slots[n] (-1: not stored). keys [pages, kv_heads, page, key_dim]; values [pages, kv_heads, value_dim, page]."""
+    n, width, ld = _rows(src, "src")
+    page = keys.shape[2]
+    _need(keys.is_contiguous() and values.is_contiguous() and keys.dtype == src.dtype == values.dtype, "cache and source types differ")
+    _need(tuple(keys.shape[1:]) == (kv_heads, page, key_dim) and tuple(values.shape[1:]) == (kv_heads, value_dim, page)
+          and values.shape[0] == keys.shape[0], "keys [pages, kv_heads, page, key_dim], values [pages, kv_heads, value_dim, page]")
+    _need(k_col + kv_heads * key_dim <= width and v_col + kv_heads * value_dim <= width and slots.numel() == n,
+          "kv_store: columns exceed the rows, or not one slot per row")
+    check(library().tw_kv_store(dtype_id(src.dtype), _dev(src), ld, int(k_col), int(v_col), _dev(slots, torch.int32, "slots"),
+                                _dev(keys), _dev(values), n, kv_heads, key_dim, value_dim, page, _stream()), "kv_store")
+
+
+def attn_mixed(q, keys, values, block_table, q_start, kv_len, seq0, n_seqs, max_q_len, out, q_heads, kv_heads, scale,
+               window=0, talk=None, sink=None, slopes=None, out_scale=1.0, splits=1, workspace=None):
+    """Attention of sequences seq0 .. seq0 + n_seqs - 1 whose scores are mixed across heads before the softmax.
+
+    q [rows, >= q_heads * key_dim] (head h at columns h * key_dim), keys [pages, kv_heads, page, key_dim], values
+    [pages, kv_heads, value_dim, page], out [rows, q_heads * value_dim]. talk float32 [H, H] mixes the scores
+    (None: no mixing), slopes float32 [H] take slope * distance off the raw scores, sink float32 [H] adds exp(sink)
+    to the softmax's denominator. splits > 1 (one-token sequences only) cuts the keys into ranges; needs a workspace.
+    """
+    key_dim, value_dim, page = keys.shape[3], values.shape[2], keys.shape[2]
+    nq, wq, ldq = _rows(q, "q")
+    no, wo, ldo = _rows(out, "out")
+    _need(wq >= q_heads * key_dim and wo == q_heads * value_dim and no == nq, "attention q/out shapes do not agree")
+    _need(out.dtype == q.dtype == keys.dtype == values.dtype, "attention operand types differ")
+    _need(keys.dim() == 4 and values.dim() == 4 and keys.is_contiguous() and values.is_contiguous()
+          and keys.shape[1] == kv_heads and tuple(values.shape[:2]) == tuple(keys.shape[:2]) and values.shape[3] == page,
+          "keys [pages, kv_heads, page, key_dim] and values [pages, kv_heads, value_dim, page] are needed")
+    _need(block_table.dim() == 2 and block_table.stride(1) == 1, "block_table must be 2-D")
+    _need(seq0 + n_seqs <= kv_len.numel() and seq0 + n_seqs <= block_table.shape[0] and q_start.numel() >= seq0 + n_seqs + 1,
+          "sequence range exceeds the metadata")
+    for name, t, count in (("talk", talk, q_heads * q_heads), ("sink", sink, q_heads), ("slopes", slopes, q_heads)):
+        _need(t is None or (t.dtype == torch.float32 and t.is_contiguous() and t.numel() == count), f"{name} has the wrong size or type")
+    ws_ptr, ws_floats = None, 0
+    if splits > 1:
+        _need(workspace is not None and workspace.dtype == torch.float32, "split attention needs a float32 workspace")
+        ws_ptr, ws_floats = _dev(workspace), workspace.numel()
+    check(library().tw_attn_mixed(dtype_id(q.dtype), _dev(q), ldq, _dev(keys), _dev(values),
+                                  _dev(block_table, torch.int32, "block_table"), block_table.stride(0),
+                                  _dev(q_start, torch.int32, "q_start"), _dev(kv_len, torch.int32, "kv_len"), int(seq0),
+                                  int(n_seqs), int(max_q_len), _dev(out), ldo,
+                                  _dev(talk) if talk is not None else None, _dev(sink) if sink is not None else None,
+                                  _dev(slopes) if slopes is not None else None, ws_ptr, ws_floats, q_heads, kv_heads,
+                                  key_dim, value_dim, page, int(window or 0), float(scale), float(out_scale), int(splits),
+                                  _stream()), "attn_mixed")
+    return out

@@ -1,15 +1,20 @@
 from .base import (Block, FeedForward, GroupStep, HeadHook, LayerRun, Mixer, Norm, Part, PositionEncoding,
                    StepContext, Workspace, fold_pending)
-from .linear import Linear
+from .linear import JoinedLinear, Linear
 from .norms import RMSNorm
 from .positions import NoPositionEncoding, RotaryEmbedding
 from .attention import GroupedQueryAttention
-from .feedforward import SwiGLU
-from .blocks import PreNormBlock
-from .embedding import OutputHead, TokenEmbedding
+from .feedforward import GatedFeedForward, SwiGLU
+from .blocks import DepthMixedBlock, PreNormBlock
+from .embedding import OutputHead, PositionedEmbedding, TokenEmbedding
+from .convolution import CausalConv
+from .parallel import GatedLinearRecurrence, MixedHeadAttention, MixerBranch, ParallelMixer
+from .side_input import SideTable, TokenSideInput
 from .model import DecoderModel, walk
 
 __all__ = ["Block", "FeedForward", "GroupStep", "HeadHook", "LayerRun", "Mixer", "Norm", "Part", "PositionEncoding",
            "StepContext", "Workspace", "fold_pending", "Linear", "RMSNorm", "NoPositionEncoding", "RotaryEmbedding",
            "GroupedQueryAttention", "SwiGLU", "PreNormBlock", "OutputHead", "TokenEmbedding",
+           "JoinedLinear", "GatedFeedForward", "DepthMixedBlock", "PositionedEmbedding", "CausalConv",
+           "GatedLinearRecurrence", "MixedHeadAttention", "MixerBranch", "ParallelMixer", "SideTable", "TokenSideInput",
            "DecoderModel", "walk"]

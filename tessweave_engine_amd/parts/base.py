@@ -125,6 +125,11 @@ class FeedForward(Part):
 class Block(Part):
     mixer: Mixer
 
+    def cache_need(self):
+        """What the block keeps per request in its cache slot: its mixer's need, unless the block itself
+        carries something more from token to token."""
+        return self.mixer.cache_need()
+
     def forward(self, ctx, run, x, pending=None):
         """Run the block on X in place. PENDING: partial sums the block before left to be added
         into X; returns what this block leaves pending (or None)."""
@@ -202,6 +207,8 @@ class StepContext:
         self.q_start = None          # int32 [n_seqs + 1]
         self.kv_len = None           # int32 [n_seqs], this step's tokens included
         self.state_slots = None      # int32 [n_seqs]
+        self.state_phase = None      # int32 [n_seqs]: which of two copies of a double-buffered state is current (the
+                                     # step reads that copy and writes the other; it alternates with every step of a request)
         self.logit_rows = None       # int32 [n_logits]
         self.n_logits = 0
         self.groups = []             # GroupStep per cache group

@@ -4,6 +4,11 @@
 """
 from __future__ import annotations
 
+import torch
+
+from ..cache.spec import CacheNeed
+from ..kernels import ops
+from ..weights.spec import NORMAL, VECTOR, TensorSpec
 from .base import Block, fold_pending
 
 
@@ -36,3 +41,69 @@ def normalise(norm, ctx, x, pending=None, rows=None):
     if pending is not None:
         return norm.forward(ctx, x, rows=rows, add=pending)
     return norm.forward(ctx, x, rows=rows)
+
+
+class DepthMixedBlock(Block):
+    """Pre-norm block whose sublayers read their normed input through a short causal convolution, with an
+    optional per-layer token input, and whose output is a learned mix of every layer's result so far:
+
+        x <- x + mixer(conv1(norm1(x)));  x <- x + ff(conv2(norm2(x)))        (the residual multiplier is the
+        x <- x + mult * side(x) / rms(side(x)) * w                              mixer's and feed-forward's own)
+        X_(layer + 1) = x;  x <- sum_{j <= layer + 1} mix[j] * X_j             (X_0 the embedding output)
+
+    mixer_in, ffn_in: `CausalConv` parts with a norm (norm, convolution and rounding are one kernel); their last
+    inputs are state of the block's cache slot beside the mixer's own. ffn / ffn_in / side / mix_name may be None.
+    The results X_j of a step live in one float32 scratch buffer [layers + 1, largest step's rows, hidden]
+    (`HISTORY_TAG`); X_0 is written there by the embedding (`PositionedEmbedding(keep=(HISTORY_TAG, layers + 1))`).
+    """
+
+    HISTORY_TAG = "depth.history"
+
+    def __init__(self, layer, n_layers, hidden, mixer_in, mixer, ffn_in=None, ffn=None, side=None, side_mult=1.0,
+                 mix_name=None):
+        self.layer, self.n_layers, self.hidden = int(layer), int(n_layers), int(hidden)
+        self.mixer_in, self.mixer, self.ffn_in, self.ffn, self.side = mixer_in, mixer, ffn_in, ffn, side
+        self.side_mult, self.mix_name = float(side_mult), mix_name
+        self.mix = None
+
+    def parts(self):
+        return [p for p in (self.mixer_in, self.mixer, self.ffn_in, self.ffn, self.side) if p is not None]
+
+    def tensor_specs(self):
+        specs = [s for p in self.parts() for s in p.tensor_specs()]
+        if self.mix_name:
+            specs.append(TensorSpec(self.mix_name, (self.layer + 2,), VECTOR, NORMAL))
+        return specs
+
+    def bind(self, tensors, dtype, device):
+        for p in self.parts():
+            p.bind(tensors, dtype, device)
+        if self.mix_name:
+            self.mix = tensors.pop(self.mix_name).contiguous()
+
+    def weight_tensors(self):
+        return [self.mix] if self.mix is not None else []
+
+    def cache_need(self):
+        need = self.mixer.cache_need() or CacheNeed()
+        own = tuple(p.state_need() for p in (self.mixer_in, self.ffn_in) if p is not None)
+        return need.merged(CacheNeed(states=own))
+
+    def forward(self, ctx, run, x, pending=None):
+        pending = fold_pending(x, pending)
+        n = ctx.n_tokens
+        h = ctx.scratch("norm.out", (n, self.hidden))
+        self.mixer_in.forward(ctx, run, x, out=h)
+        self.mixer.forward(ctx, run, h, x)
+        if self.ffn is not None:
+            self.ffn_in.forward(ctx, run, x, out=h)
+            self.ffn.forward(ctx, h, x)
+        y = self.side.forward(ctx, x) if self.side is not None else None
+        history = None
+        if self.mix is not None:
+            history = ctx.workspace.get(self.HISTORY_TAG, (self.n_layers + 1, ctx.max_tokens, self.hidden), torch.float32)
+        if y is not None or history is not None:
+            ops.layer_end(x, self.layer, branch=y, branch_weight=self.side.weight if self.side is not None else None,
+                          eps=self.side.eps if self.side is not None else 0.0, mult=self.side_mult, history=history,
+                          mix=self.mix)
+        return None

@@ -38,3 +38,40 @@ class SwiGLU(FeedForward):
             return self.down.forward_partials(ctx, act, "down")
         self.down.forward(ctx, act, x, residual=x)
         return None
+
+
+class GatedFeedForward(FeedForward):
+    """x += out_scale * down( act(gate(h)) * up(h) ) with a choice of activation and of tensor names.
+
+    activation "silu" is `SwiGLU`'s arithmetic; "gelu_tanh" is 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))).
+    The gelu form multiplies in a kernel of its own after one packed gate|up product (the fused epilogue of the
+    matrix kernels is SiLU's); out_scale is folded into that multiplication, before the rounding to the compute
+    type, so the down projection adds straight into the residual stream.
+    """
+
+    def __init__(self, names, hidden, intermediate, activation="gelu_tanh", out_scale=1.0, suffix=".weight"):
+        if activation != "gelu_tanh":
+            raise ValueError("GatedFeedForward computes gelu_tanh; SwiGLU is the SiLU part")
+        gate, up, down = names
+        self.hidden, self.intermediate, self.out_scale = int(hidden), int(intermediate), float(out_scale)
+        self.gate_up = Linear([gate, up], hidden, [intermediate, intermediate], suffixes=(suffix, ".bias"))
+        self.down = Linear([down], intermediate, [hidden], suffixes=(suffix, ".bias"))
+
+    def parts(self):
+        return [self.gate_up, self.down]
+
+    def tensor_specs(self):
+        return self.gate_up.tensor_specs() + self.down.tensor_specs()
+
+    def bind(self, tensors, dtype, device):
+        self.gate_up.bind(tensors, dtype, device)
+        self.down.bind(tensors, dtype, device)
+
+    def forward(self, ctx, h, x):
+        n = h.shape[0]
+        gu = ctx.scratch("ffn.gate_up", (n, 2 * self.intermediate))
+        self.gate_up.forward(ctx, h, gu)
+        act = ctx.scratch("ffn.act", (n, self.intermediate))
+        ops.gelu_mul(gu, act, self.out_scale)
+        self.down.forward(ctx, act, x, residual=x)
+        return None

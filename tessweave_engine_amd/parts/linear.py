@@ -27,7 +27,7 @@ def pad_groups(t, dim, unit, to):
 
 class Linear(Part):
     def __init__(self, names, in_features, out_features, bias=False, packed=True, glu=False,
-                 pad_out=None, pad_in=None):
+                 pad_out=None, pad_in=None, suffixes=(".weight", ".bias")):
         """names[i] is the checkpoint prefix of the i-th matrix ("...q_proj"), out_features[i] its rows.
 
         glu: the two matrices are a gate and an up projection; if they can be packed with their
@@ -36,18 +36,47 @@ class Linear(Part):
         `to - unit` rows of zeros (and zero biases), so the layer's output has groups of `to` columns
         whose tail is exactly zero. pad_in = (unit, to): the same for groups of input columns (the
         input then has groups of `to` columns, whose tails meet zeros). The checkpoint's tensors keep
-        their own shapes.
+        their own shapes. pad_out may also be a list with one (unit, to) or None per matrix, and pad_in a
+        list of (columns, unit, to) runs that together cover the input (several inputs side by side, each
+        with its own groups).
+        bias may be a list with one flag per matrix: a matrix without one gets zeros on the device.
+        suffixes: what a matrix's name is followed by in the checkpoint for its weight and its bias.
         """
         self.names = list(names)
         self.in_features = int(in_features)
         self.out_features = [int(o) for o in out_features]
-        self.has_bias = bool(bias)
+        self.bias_flags = [bool(b) for b in bias] if isinstance(bias, (list, tuple)) else [bool(bias)] * len(self.names)
+        if len(self.bias_flags) != len(self.names):
+            raise ValueError("one bias flag per matrix is needed")
+        self.has_bias = any(self.bias_flags)
+        self.suffixes = tuple(suffixes)
         self.packed = bool(packed)
         self.glu = bool(glu)
-        self.pad_out = tuple(int(v) for v in pad_out) if pad_out and pad_out[0] != pad_out[1] else None
-        self.pad_in = tuple(int(v) for v in pad_in) if pad_in and pad_in[0] != pad_in[1] else None
-        for pad, sizes in ((self.pad_out, self.out_features), (self.pad_in, [self.in_features])):
-            if pad and (pad[1] < pad[0] or any(n % pad[0] for n in sizes)):
+
+        def pair(p):
+            return tuple(int(v) for v in p) if p and p[0] != p[1] else None
+        if pad_out and isinstance(pad_out[0], (list, tuple, type(None))):
+            self.pad_outs = [pair(p) for p in pad_out]
+        else:
+            self.pad_outs = [pair(pad_out)] * len(self.names)
+        if len(self.pad_outs) != len(self.names):
+            raise ValueError("one output padding per matrix is needed")
+        self.pad_out = self.pad_outs[0] if len(set(self.pad_outs)) == 1 else None
+        if pad_in and isinstance(pad_in[0], (list, tuple)):
+            self.pad_ins = [tuple(int(v) for v in run) for run in pad_in]
+            if sum(run[0] for run in self.pad_ins) != self.in_features:
+                raise ValueError("the input's padded runs must cover its columns")
+            if all(u == t for _, u, t in self.pad_ins):
+                self.pad_ins = None
+        else:
+            single = pair(pad_in)
+            self.pad_ins = [(self.in_features, *single)] if single else None
+        self.pad_in = pair(pad_in) if not (pad_in and isinstance(pad_in[0], (list, tuple))) else None
+        for pad, rows in zip(self.pad_outs, self.out_features):
+            if pad and (pad[1] < pad[0] or rows % pad[0]):
+                raise ValueError("padded groups must divide the layer's sizes and may only grow")
+        for columns, unit, to in self.pad_ins or []:
+            if to < unit or columns % unit:
                 raise ValueError("padded groups must divide the layer's sizes and may only grow")
         self.gated = False
         self.weights = []       # one tensor if packed, else one per name
@@ -60,20 +89,42 @@ class Linear(Part):
 
     def tensor_specs(self):
         specs = []
-        for name, rows in zip(self.names, self.out_features):
-            specs.append(TensorSpec(name + ".weight", (rows, self.in_features), MATRIX, NORMAL))
-            if self.has_bias:
-                specs.append(TensorSpec(name + ".bias", (rows,), VECTOR, NORMAL))
+        for name, rows, flag in zip(self.names, self.out_features, self.bias_flags):
+            specs.append(TensorSpec(name + self.suffixes[0], (rows, self.in_features), MATRIX, NORMAL))
+            if flag:
+                specs.append(TensorSpec(name + self.suffixes[1], (rows,), VECTOR, NORMAL))
         return specs
 
+    @property
+    def device_in(self):
+        """Input columns on the device (padded groups included)."""
+        if not self.pad_ins:
+            return self.in_features
+        return sum(columns // unit * to for columns, unit, to in self.pad_ins)
+
+    @property
+    def device_out(self):
+        """Output columns of each matrix on the device (padded groups included)."""
+        return [rows // pad[0] * pad[1] if pad else rows for rows, pad in zip(self.out_features, self.pad_outs)]
+
     def bind(self, tensors, dtype, device):
-        weights = [tensors.pop(name + ".weight") for name in self.names]
-        biases = [tensors.pop(name + ".bias") for name in self.names] if self.has_bias else []
-        if self.pad_out:
-            weights = [pad_groups(w, 0, *self.pad_out) for w in weights]
-            biases = [pad_groups(b, 0, *self.pad_out) for b in biases]
-        if self.pad_in:
-            weights = [pad_groups(w, 1, *self.pad_in) for w in weights]
+        weights = [tensors.pop(name + self.suffixes[0]) for name in self.names]
+        biases = []
+        if self.has_bias:
+            biases = [tensors.pop(name + self.suffixes[1]) if flag else
+                      torch.zeros(rows, dtype=torch.float32, device=weights[0].device)
+                      for name, rows, flag in zip(self.names, self.out_features, self.bias_flags)]
+        weights = [pad_groups(w, 0, *pad) if pad else w for w, pad in zip(weights, self.pad_outs)]
+        biases = [pad_groups(b, 0, *pad) if pad else b for b, pad in zip(biases, self.pad_outs)]
+        if self.pad_ins:
+            padded = []
+            for w in weights:
+                runs, col = [], 0
+                for columns, unit, to in self.pad_ins:
+                    runs.append(pad_groups(w[:, col:col + columns], 1, unit, to))
+                    col += columns
+                padded.append(torch.cat(runs, 1) if len(runs) > 1 else runs[0])
+            weights = padded
         self.gated = (self.glu and self.packed and len(weights) == 2 and
                       weights[0].shape == weights[1].shape and weights[0].shape[0] % 16 == 0)
         if self.gated:
@@ -166,3 +217,34 @@ class Linear(Part):
             buf = ctx.workspace.get("linear.partial.rows." + tag, (splits, n, w.shape[0]), torch.float32)
         partial = buf.view(-1)[:splits * n * w.shape[0]].view(splits, n, w.shape[0])
         return ops.linear_partials(x, w, partial)
+
+
+class JoinedLinear(Linear):
+    """One product over several inputs laid side by side: out = [x_0 | x_1 | ...] @ [W_0 | W_1 | ...].T, the
+    matrices W_i [out, in_i] joined along their columns into one weight, so that the outputs of parallel
+    branches meet in one product (and one addition into the residual stream) instead of one each.
+
+    pad_ins[i] = (unit, to) or None lays groups of input i out with tails of zeros, as `Linear(pad_in=)` does.
+    """
+
+    def __init__(self, names, in_features, out_features, pad_ins=None, suffix=".weight"):
+        self.part_names = list(names)
+        self.part_in = [int(k) for k in in_features]
+        pads = list(pad_ins) if pad_ins else [None] * len(self.part_names)
+        runs = [(k, *(pad if pad else (k, k))) for k, pad in zip(self.part_in, pads)]
+        super().__init__(["|".join(self.part_names)], sum(self.part_in), [out_features], pad_in=runs,
+                         suffixes=(suffix, ".bias"))
+        self.part_runs = runs
+
+    def tensor_specs(self):
+        return [TensorSpec(name + self.suffixes[0], (self.out_features[0], k), MATRIX, NORMAL)
+                for name, k in zip(self.part_names, self.part_in)]
+
+    @property
+    def device_in_parts(self):
+        """Columns of each input on the device."""
+        return [columns // unit * to for columns, unit, to in self.part_runs]
+
+    def bind(self, tensors, dtype, device):
+        joined = torch.cat([tensors.pop(name + self.suffixes[0]) for name in self.part_names], 1)
+        super().bind({self.names[0] + self.suffixes[0]: joined}, dtype, device)

@@ -91,13 +91,13 @@ class DecoderModel(Part):
             n_slots = max((run.cache_slot for run in self.schedule), default=-1) + 1
             needs = [None] * n_slots
             for run in self.schedule:
-                need = self.blocks[run.block].mixer.cache_need()
+                need = self.blocks[run.block].cache_need()
                 if run.writes_cache:
                     if needs[run.cache_slot] is not None and needs[run.cache_slot] != need:
                         raise ValueError(f"cache slot {run.cache_slot} is written with two different needs")
                     needs[run.cache_slot] = need
             for run in self.schedule:
-                need = self.blocks[run.block].mixer.cache_need()
+                need = self.blocks[run.block].cache_need()
                 if not run.writes_cache and needs[run.cache_slot] != need:
                     raise ValueError(f"a layer reads cache slot {run.cache_slot}, which holds something else")
             self._layout = CacheLayout(needs)

@@ -14,17 +14,18 @@ from .base import Norm
 class RMSNorm(Norm):
     folds_pending = True
 
-    def __init__(self, name, size, eps):
+    def __init__(self, name, size, eps, suffix=".weight"):
         self.name = name
+        self.suffix = suffix              # what follows the name in the checkpoint
         self.size = int(size)
         self.eps = float(eps)
         self.weight = None
 
     def tensor_specs(self):
-        return [TensorSpec(self.name + ".weight", (self.size,), VECTOR, ONE_PLUS_NORMAL)]
+        return [TensorSpec(self.name + self.suffix, (self.size,), VECTOR, ONE_PLUS_NORMAL)]
 
     def bind(self, tensors, dtype, device):
-        self.weight = tensors.pop(self.name + ".weight").contiguous()
+        self.weight = tensors.pop(self.name + self.suffix).contiguous()
 
     def weight_tensors(self):
         return [self.weight]
