@@ -112,7 +112,8 @@ def attention_branch(h, w, p, spec):
     q = (h @ w[p + "q"].T).view(T, H, D)
     k = (h @ w[p + "k"].T).view(T, G, D)
     v = (h @ w[p + "v"].T).view(T, G, E)
-    o = mixed_head_attention(q, k, v, spec["scale"], spec["mask"]["size"], w[p + "talk"], w[p + "sink"])
+    window = spec["mask"]["size"] if spec.get("mask") else T + 1          # no mask entry: every earlier key is seen
+    o = mixed_head_attention(q, k, v, spec["scale"], window, w[p + "talk"], w[p + "sink"])
     return o.reshape(T, H * E) @ w[p + "o"].T
 
 
@@ -154,7 +155,8 @@ def forward(config, weights, tokens, dtype=torch.float64, layers_out=None):
         if layer.get("mlp"):
             h = input_conv(rms_norm(x, w[p + "norm2"], eps), w[p + "canon2"])
             x = x + m * dense_feed_forward(h, w, p + "mlp.")
-        x = x + m * token_side_input(x, tokens, w, i, config["token_side"]["dim"], eps)
+        if config.get("token_side"):
+            x = x + m * token_side_input(x, tokens, w, i, config["token_side"]["dim"], eps)
         results.append(x)
         if layers_out is not None:
             layers_out.append(x)
