@@ -19,7 +19,9 @@ as the weights; `prefill_32k_prompts`: tokens a second over those prompts, which
 go through in portions of 2,048); and 1,024-token prompts with 512 generated tokens at batch 1, 8 and 64
 (`gen512_b*`, decoded tokens a second over the generated part).
 
-Other sizes of the architecture: --shape 14b|32b. --serve measures continuous
+Other sizes of the architecture: --shape 14b|32b. --design kanavik measures the Kanavik
+design's prefill and decode at a few layer sizes, each beside the Qwen2 decoder at equal
+width, heads, feed-forward and depth (one JSON line a size). --serve measures continuous
 batching under Poisson arrivals instead (prompts of 128..4,096 tokens, 256
 generated tokens each, prompt portions of 512) and prints its own JSON line.
 """
@@ -87,7 +89,71 @@ def parse():
                    help="with --serve: the largest prompt portion in one step (larger: more prompt tokens a second and "
                         "a shorter time to the first token, longer steps for the requests that are decoding)")
     p.add_argument("--rate", type=float, default=16.0, help="mean arrivals a second (0: all at once)")
+    p.add_argument("--design", default="", choices=["", "kanavik"],
+                   help="instead: prefill and decode throughput of another design at a few layer sizes (--design-sizes), "
+                        "each beside the Qwen2 decoder at equal width, heads, feed-forward and depth; one JSON line a size")
+    p.add_argument("--design-sizes", default="1b,3b,7b", help="which of the design's sizes to run, comma separated")
+    p.add_argument("--design-layers", type=int, default=8, help="layers of every model of a --design run")
+    p.add_argument("--design-only", action="store_true", help="with --design: skip the Qwen2 model beside it (profiling runs)")
     return p.parse_args()
+
+
+# Layer sizes for --design runs: (width, query heads, key/value heads, head size, feed-forward, window)
+DESIGN_SIZES = {"1b": (2048, 16, 4, 128, 5632, 1024), "3b": (3072, 24, 4, 128, 8192, 2048), "7b": (4096, 32, 8, 128, 11008, 4096)}
+DESIGN_VOCAB = 32000
+
+
+def kanavik_config(size, layers, context):
+    width, heads, kv_heads, dim, ff, window = DESIGN_SIZES[size]
+    layer = {"type": "parallel",
+             "mixer": {"left": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+                                "mask": {"size": window}},
+                       "right": {"width": width, "blocks": 16, "conv": 4}, "left_scale": 1.0, "right_scale": 1.0},
+             "mlp": {"kind": "dense", "ff": ff}}
+    return {"architecture": "Kanavik", "vocab": DESIGN_VOCAB, "width": width, "max_positions": max(8192, context + 1),
+            "norm": {"eps": 1e-6}, "residual_mult": 1.0, "canon": {"taps": 4}, "token_side": {"dim": 128},
+            "layers": [layer] * layers}
+
+
+def qwen2_config_like(size, layers, context):
+    width, heads, kv_heads, dim, ff, _ = DESIGN_SIZES[size]
+    return dict(QWEN25_7B, num_hidden_layers=layers, hidden_size=width, num_attention_heads=heads,
+                num_key_value_heads=kv_heads, head_dim=dim, intermediate_size=ff, vocab_size=DESIGN_VOCAB,
+                max_position_embeddings=max(8192, context + 1))
+
+
+def design_run(args, torch):
+    """One JSON line a size: the design's prefill and decode throughput and, beside it, the Qwen2 decoder's at equal
+    width, heads, feed-forward size and depth (same engine, same scheduler, random weights)."""
+    from tessweave_engine_amd.config import config_from_dict
+    from tessweave_engine_amd.weights import random_model
+    use_graphs = not args.no_graphs
+    steps, warmup = min(args.steps, 64), min(args.warmup, 8)
+    for size in [v for v in args.design_sizes.split(",") if v]:
+        line = {"design": args.design, "size": size, "layers": args.design_layers, "dtype": args.dtype,
+                "sizes": dict(zip(("width", "heads", "kv_heads", "head_dim", "ff", "window"), DESIGN_SIZES[size])),
+                "batch": args.batch, "context": args.context, "prefill_tokens": args.prefill_tokens,
+                "data": "synthetic: uniform-random token ids, random weights"}
+        models = [(args.design, kanavik_config(size, args.design_layers, args.context))]
+        if not args.design_only:
+            models.append(("qwen2", qwen2_config_like(size, args.design_layers, args.context)))
+        for name, cfg in models:
+            model = random_model(config_from_dict(cfg), args.seed, dtype=args.dtype, device="cuda:0")
+            entry = {"weight_gb": round(model.weight_bytes() / 1e9, 3)}
+            if args.prefill_tokens > 0:
+                ms = prefill_run(model, torch, args.prefill_tokens, args.dtype, args.seed)
+                entry.update(prefill_ms=round(ms, 3), prefill_tokens_per_s=round(args.prefill_tokens / (ms / 1000), 1))
+            if not args.prefill_only:
+                tps, ms_step, replays, _ = decode_run(model, torch, args.batch, args.context, steps, warmup, args.dtype,
+                                                      use_graphs, args.seed)
+                entry.update(decode_tokens_per_s=round(tps, 1), decode_ms_per_step=round(ms_step, 4),
+                             decode_weight_read_gbs=round(model.weight_bytes() / (ms_step / 1000) / 1e9, 1),
+                             graph_replays=replays)
+            line[name] = entry
+            del model
+            torch.cuda.empty_cache()
+        print(json.dumps(line), flush=True)
+    return 0
 
 
 def decode_run(model, torch, batch, context, steps, warmup, dtype, use_graphs, seed, max_context=0):
@@ -317,6 +383,8 @@ def main():
     from tessweave_engine_amd.config import config_from_dict
     from tessweave_engine_amd.weights import random_model
 
+    if args.design:
+        return design_run(args, torch)
     shape_name, sizes = SHAPES[args.shape]
     cfg = dict(QWEN25_7B, **sizes)
     layers_full = cfg["num_hidden_layers"]

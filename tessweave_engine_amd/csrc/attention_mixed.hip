@@ -278,15 +278,16 @@ static int mixed_launch(const MixedAttnArgs& a, int n_seqs, int tiles, int waves
 template <typename T>
 static int mixed_dispatch(const MixedAttnArgs& a, int n_seqs, int max_q_len, hipStream_t stream) {
   const int tiles = tw_div_up(max_q_len, 16);
-  // One head a wave up to 16 heads; two a wave (values of up to 64 elements only: the output sums of a
+  // One head a wave up to 16 heads; two a wave (values of up to 128 elements only: the output sums of a
   // wave's heads live in its registers) up to 32.
   const int hpw = a.H <= 16 ? 1 : 2;
   const int waves = tw_div_up(a.H, hpw);
   const size_t lds = mx_lds_bytes<T>(a.H, a.D);
-  TW_REQUIRE(waves <= 16 && lds <= 150 * 1024 && (hpw == 1 || a.E <= 64));
+  TW_REQUIRE(waves <= 16 && lds <= 150 * 1024 && (hpw == 1 || a.E <= 128));
   int code;
   if (hpw == 2)
-    code = mixed_launch<T, 2, 4>(a, n_seqs, tiles, waves, lds, stream);
+    code = a.E <= 64 ? mixed_launch<T, 2, 4>(a, n_seqs, tiles, waves, lds, stream)
+                     : mixed_launch<T, 2, 8>(a, n_seqs, tiles, waves, lds, stream);
   else if (a.E <= 64)
     code = mixed_launch<T, 1, 4>(a, n_seqs, tiles, waves, lds, stream);
   else if (a.E <= 128)

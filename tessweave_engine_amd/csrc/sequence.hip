@@ -76,7 +76,7 @@ struct ConvArgs {
 
 template <typename SrcT, typename OutT, bool NORM>
 __global__ __launch_bounds__(256) void causal_conv_kernel(ConvArgs a) {
-  __shared__ float red[16];
+  __shared__ float red[TW_CONV_MAX_TAPS][4];
   __shared__ float rinv[TW_CONV_MAX_TAPS];
   const int row = blockIdx.x;
   const int s = tw_seq_of_row(a.q_start, a.n_seqs, row);
@@ -90,38 +90,63 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(ConvArgs a) {
   float* new_state = a.state + ((size_t)slot * 2 + (1 - ph)) * (size_t)(K - 1) * C;
   const bool last = pos == len - 1;
   const SrcT* src = (const SrcT*)a.src;
-
+  // where each tap's row comes from: this step's rows, the state, or nothing (the same for the whole block)
+  const SrcT* from_src[TW_CONV_MAX_TAPS];
+  const float* from_state[TW_CONV_MAX_TAPS];
+#pragma unroll
+  for (int j = 0; j < TW_CONV_MAX_TAPS; ++j) {
+    const int p = pos - (K - 1) + j;
+    from_src[j] = (j < K && p >= start) ? src + (size_t)(first + p - start) * a.ld_src : nullptr;
+    from_state[j] = (j < K && p < start && p >= 0) ? old_state + (size_t)(p - start + K - 1) * C : nullptr;
+  }
   if (NORM) {
-    for (int j = 0; j < K; ++j) {
-      const int p = pos - (K - 1) + j;
-      float sum = 0.f;
-      if (p >= start) {
-        const SrcT* r = src + (size_t)(first + p - start) * a.ld_src;
-        for (int c = threadIdx.x; c < C; c += blockDim.x) {
-          const float v = tw_to_float(r[c]);
-          sum += v * v;
+    // every block sums whole rows, whatever share of the channels it then writes
+    float sums[TW_CONV_MAX_TAPS];
+#pragma unroll
+    for (int j = 0; j < TW_CONV_MAX_TAPS; ++j) sums[j] = 0.f;
+    for (int c = threadIdx.x; c < C; c += blockDim.x) {
+#pragma unroll
+      for (int j = 0; j < TW_CONV_MAX_TAPS; ++j)
+        if (from_src[j]) {
+          const float v = tw_to_float(from_src[j][c]);
+          sums[j] += v * v;
         }
+    }
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+#pragma unroll
+    for (int j = 0; j < TW_CONV_MAX_TAPS; ++j) {
+      if (j < K) {
+        const float t = tw_wave_sum(sums[j]);
+        if (lane == 0) red[j][wave] = t;
       }
-      sum = tw_block_sum(sum, red);
-      if (threadIdx.x == 0) rinv[j] = rsqrtf(sum / (float)C + a.eps);
+    }
+    __syncthreads();
+    if (threadIdx.x < K) {
+      const int j = threadIdx.x;
+      rinv[j] = rsqrtf((red[j][0] + red[j][1] + red[j][2] + red[j][3]) / (float)C + a.eps);
     }
     __syncthreads();
   }
-  for (int c = threadIdx.x; c < C; c += blockDim.x) {
+  const int share = (C + gridDim.y - 1) / gridDim.y;
+  const int c_end = min(C, (int)(blockIdx.y + 1) * share);
+  for (int c = blockIdx.y * share + threadIdx.x; c < c_end; c += blockDim.x) {
+    float v[TW_CONV_MAX_TAPS];
+#pragma unroll
+    for (int j = 0; j < TW_CONV_MAX_TAPS; ++j) {
+      v[j] = 0.f;
+      if (from_src[j]) v[j] = tw_to_float(from_src[j][c]);
+      else if (from_state[j]) v[j] = from_state[j][c];
+    }
     float acc = a.bias ? a.bias[c] : 0.f;
     const float nw = NORM ? a.norm_w[c] : 1.f;
-    for (int j = 0; j < K; ++j) {
-      const int p = pos - (K - 1) + j;
-      float v = 0.f;
-      if (p >= start) {
-        v = tw_to_float(src[(size_t)(first + p - start) * a.ld_src + c]);
-        if (NORM) v = v * rinv[j] * nw;
-      } else if (p >= 0) {
-        v = old_state[(size_t)(p - start + K - 1) * C + c];
+#pragma unroll
+    for (int j = 0; j < TW_CONV_MAX_TAPS; ++j) {
+      if (j < K) {
+        if (NORM && from_src[j]) v[j] = v[j] * rinv[j] * nw;
+        acc += a.taps[(size_t)c * K + j] * v[j];
+        if (j == K - 1) acc += a.identity * v[j];
+        if (last && j >= 1) new_state[(size_t)(j - 1) * C + c] = v[j];
       }
-      acc += a.taps[(size_t)c * K + j] * v;
-      if (j == K - 1) acc += a.identity * v;
-      if (last && j >= 1) new_state[(size_t)(j - 1) * C + c] = v;
     }
     if (a.out) ((OutT*)a.out)[(size_t)row * a.ld_out + c] = tw_from_float<OutT>(acc);
     if (a.out32) a.out32[(size_t)row * a.ld_out32 + c] = acc;
@@ -144,15 +169,19 @@ extern "C" int tw_causal_conv(int dtype, int src_f32, const void* src, long ld_s
              out, ld_out, out32, ld_out32, n_seqs, C, K, eps, identity};
   const bool bf = dtype == TW_DTYPE_BF16;
   TW_REQUIRE(bf || dtype == TW_DTYPE_F32);
+  // few rows (decode steps): the channels are shared out over several blocks a row
+  int shares = n_tokens >= 512 ? 1 : tw_div_up(C, 512);
+  if (shares > 8) shares = 8;
+  const dim3 n_blocks(n_tokens, shares);
   if (norm_w) {
-    if (bf) causal_conv_kernel<float, bf16_t, true><<<n_tokens, 256, 0, stream>>>(a);
-    else causal_conv_kernel<float, float, true><<<n_tokens, 256, 0, stream>>>(a);
+    if (bf) causal_conv_kernel<float, bf16_t, true><<<n_blocks, 256, 0, stream>>>(a);
+    else causal_conv_kernel<float, float, true><<<n_blocks, 256, 0, stream>>>(a);
   } else if (src_f32) {
-    if (bf) causal_conv_kernel<float, bf16_t, false><<<n_tokens, 256, 0, stream>>>(a);
-    else causal_conv_kernel<float, float, false><<<n_tokens, 256, 0, stream>>>(a);
+    if (bf) causal_conv_kernel<float, bf16_t, false><<<n_blocks, 256, 0, stream>>>(a);
+    else causal_conv_kernel<float, float, false><<<n_blocks, 256, 0, stream>>>(a);
   } else {
-    if (bf) causal_conv_kernel<bf16_t, bf16_t, false><<<n_tokens, 256, 0, stream>>>(a);
-    else causal_conv_kernel<float, float, false><<<n_tokens, 256, 0, stream>>>(a);
+    if (bf) causal_conv_kernel<bf16_t, bf16_t, false><<<n_blocks, 256, 0, stream>>>(a);
+    else causal_conv_kernel<float, float, false><<<n_blocks, 256, 0, stream>>>(a);
   }
   return TW_LAUNCH_RESULT();
 }
@@ -175,49 +204,165 @@ struct RecurrenceArgs {
   void* out; long ld_out;
   int C, block_size;
   float decay, out_scale;
+  int chunk;                          // tokens a thread walks; a sequence's portion is cut into chunks of this length
+  int max_chunks;                     // chunks of the longest portion of the launch (1: no cutting, one kernel)
+  float* part;                        // max_chunks > 1: [seq][max_chunks][3][C]: product of a, state from zero, (chunk 0) state before
+  int out_pad;                        // columns [C, C + out_pad) of out are set to zero
 };
 
-template <typename T>
+// One step of the recurrence for channel c at token t; returns a_t and adds into S.
+__device__ __forceinline__ float recurrence_step(const RecurrenceArgs& a, int t, int c, int ga, int gi, float unit, float& S) {
+  const float r = tw_sigmoid(a.gates[(size_t)t * a.ld_gates + ga]);
+  const float i = tw_sigmoid(a.gates[(size_t)t * a.ld_gates + gi]);
+  const float la = -unit * r;
+  const float dec = expf(la);
+  const float norm = sqrtf(fmaxf(0.f, -expm1f(2.f * la)));          // sqrt(1 - a^2) without cancellation
+  S = dec * S + norm * i * a.u[(size_t)t * a.ld_u + c];
+  return dec;
+}
+
+// FINAL false: a chunk's product of decays and its state from zero (and, chunk 0, the state before the step) go
+// to `part`. FINAL true: the chunk's true start state is rebuilt from the chunks before it, the chunk is walked
+// again and the outputs are written; the sequence's last chunk leaves the new state. A portion of one chunk
+// (every decode step) needs the FINAL kernel only and reads the state itself.
+template <typename T, bool FINAL>
 __global__ __launch_bounds__(256) void gated_recurrence_kernel(RecurrenceArgs a) {
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
-  if (c >= a.C) return;
-  const int s = blockIdx.y;
+  const int s = blockIdx.y, z = blockIdx.z;
   const int first = a.q_start[s], end = a.q_start[s + 1];
+  const int n_chunks = (end - first + a.chunk - 1) / a.chunk;
+  if (z >= n_chunks) return;
+  const int t0 = first + z * a.chunk, t1 = min(end, t0 + a.chunk);
+  T* out = (T*)a.out;
+  if (FINAL && c >= a.C) {
+    if (c < a.C + a.out_pad)
+      for (int t = t0; t < t1; ++t) out[(size_t)t * a.ld_out + c] = tw_from_float<T>(0.f);
+    return;
+  }
+  if (c >= a.C) return;
   float* st = a.state + (size_t)a.state_slots[s] * a.C + c;
-  float S = *st;
   const float lam = a.lam[c];
   const float unit = a.decay * (lam > 20.f ? lam : log1pf(expf(lam)));
   const int b = c / a.block_size, k = c % a.block_size;
   const int ga = 2 * b * a.block_size + k, gi = ga + a.block_size;
+  float* part = a.part ? a.part + ((size_t)s * a.max_chunks) * 3 * a.C + c : nullptr;
+  if (!FINAL) {
+    if (n_chunks == 1) return;
+    float S = 0.f, P = 1.f;
+    for (int t = t0; t < t1; ++t) P *= recurrence_step(a, t, c, ga, gi, unit, S);
+    part[((size_t)z * 3 + 0) * a.C] = P;
+    part[((size_t)z * 3 + 1) * a.C] = S;
+    if (z == 0) part[2 * (size_t)a.C] = *st;
+    return;
+  }
+  float S;
+  if (n_chunks == 1) {
+    S = *st;
+  } else {
+    S = part[2 * (size_t)a.C];
+    for (int j = 0; j < z; ++j) S = part[((size_t)j * 3 + 0) * a.C] * S + part[((size_t)j * 3 + 1) * a.C];
+  }
   const T* branch = (const T*)a.branch;
-  T* out = (T*)a.out;
-  for (int t = first; t < end; ++t) {
-    const float r = tw_sigmoid(a.gates[(size_t)t * a.ld_gates + ga]);
-    const float i = tw_sigmoid(a.gates[(size_t)t * a.ld_gates + gi]);
-    const float la = -unit * r;
-    const float dec = expf(la);
-    const float norm = sqrtf(fmaxf(0.f, -expm1f(2.f * la)));          // sqrt(1 - a^2) without cancellation
-    S = dec * S + norm * i * a.u[(size_t)t * a.ld_u + c];
+  for (int t = t0; t < t1; ++t) {
+    recurrence_step(a, t, c, ga, gi, unit, S);
     const float y = tw_gelu_tanh(tw_to_float(branch[(size_t)t * a.ld_branch + c]));
     out[(size_t)t * a.ld_out + c] = tw_from_float<T>(a.out_scale * S * y);
   }
-  *st = S;
+  if (z == n_chunks - 1) *st = S;
+}
+
+#define TW_RECURRENCE_CHUNK 64
+
+extern "C" long tw_gated_recurrence_workspace_floats(int n_seqs, int max_q_len, int C) {
+  const int chunks = tw_div_up(max_q_len, TW_RECURRENCE_CHUNK);
+  return chunks > 1 ? (long)n_seqs * chunks * 3 * C : 0;
 }
 
 extern "C" int tw_gated_recurrence(int dtype, const float* gates, long ld_gates, const float* u, long ld_u,
                                    const void* branch, long ld_branch, const float* lam, float* state,
                                    const int* q_start, const int* state_slots, void* out, long ld_out, int n_seqs,
-                                   int C, int blocks, float decay, float out_scale, hipStream_t stream) {
+                                   int max_q_len, int C, int blocks, int out_pad, float decay, float out_scale,
+                                   float* workspace, long workspace_floats, hipStream_t stream) {
   TW_REQUIRE(gates && u && branch && lam && state && q_start && state_slots && out);
-  TW_REQUIRE(n_seqs >= 0 && C > 0 && blocks > 0 && C % blocks == 0);
-  TW_REQUIRE(ld_gates >= 2 * C && ld_u >= C && ld_branch >= C && ld_out >= C);
+  TW_REQUIRE(n_seqs >= 0 && max_q_len >= 1 && C > 0 && blocks > 0 && C % blocks == 0 && out_pad >= 0);
+  TW_REQUIRE(ld_gates >= 2 * C && ld_u >= C && ld_branch >= C && ld_out >= C + out_pad);
   if (n_seqs == 0) return 0;
+  const int chunks = tw_div_up(max_q_len, TW_RECURRENCE_CHUNK);
+  TW_REQUIRE(chunks == 1 || (workspace && workspace_floats >= tw_gated_recurrence_workspace_floats(n_seqs, max_q_len, C)));
   RecurrenceArgs a{gates, ld_gates, u, ld_u, branch, ld_branch, lam, state, q_start, state_slots, out, ld_out,
-                   C, C / blocks, decay, out_scale};
-  dim3 grid(tw_div_up(C, 256), n_seqs);
-  if (dtype == TW_DTYPE_BF16) gated_recurrence_kernel<bf16_t><<<grid, 256, 0, stream>>>(a);
-  else if (dtype == TW_DTYPE_F32) gated_recurrence_kernel<float><<<grid, 256, 0, stream>>>(a);
-  else return TW_ERR_BAD_ARGUMENT;
+                   C, C / blocks, decay, out_scale, TW_RECURRENCE_CHUNK, chunks, chunks > 1 ? workspace : nullptr, out_pad};
+  TW_REQUIRE(dtype == TW_DTYPE_BF16 || dtype == TW_DTYPE_F32);
+  const dim3 grid_part(tw_div_up(C, 256), n_seqs, chunks), grid(tw_div_up(C + out_pad, 256), n_seqs, chunks);
+  if (chunks > 1) {
+    if (dtype == TW_DTYPE_BF16) gated_recurrence_kernel<bf16_t, false><<<grid_part, 256, 0, stream>>>(a);
+    else gated_recurrence_kernel<float, false><<<grid_part, 256, 0, stream>>>(a);
+  }
+  if (dtype == TW_DTYPE_BF16) gated_recurrence_kernel<bf16_t, true><<<grid, 256, 0, stream>>>(a);
+  else gated_recurrence_kernel<float, true><<<grid, 256, 0, stream>>>(a);
+  return TW_LAUNCH_RESULT();
+}
+
+// ---- block-diagonal product: out[n][b * No + o] = sum_i x[n][b * Ni + i] * w[b][o][i] + bias[b * No + o] ---------
+// `blocks` square-ish matrices [No][Ni] side by side along the diagonal (the gates of a recurrence read only
+// their own block of channels). One wave takes 16 rows and 64 output columns of one block: the weights are the
+// A operand (so a lane ends with 4 consecutive output columns of one row), the rows the B operand, both read
+// straight from memory in 16-byte fragments. Ni must be a multiple of 16 bytes, No of 16.
+template <typename T>
+__global__ __launch_bounds__(256) void block_diagonal_kernel(const T* __restrict__ x, long ldx, const T* __restrict__ w,
+                                                             const float* __restrict__ bias, float* __restrict__ out,
+                                                             long ldo, int n, int blocks, int Ni, int No, int col_groups) {
+  typedef typename Elem<T>::Frag Frag;
+  constexpr int EPF = Elem<T>::kPerFrag;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int unit = blockIdx.x * 4 + wave;                  // (block, group of 64 columns)
+  const int b = unit / col_groups, cg = unit % col_groups;
+  if (b >= blocks) return;
+  const int row0 = blockIdx.y * 16;
+  const int chunks = Ni / EPF, steps = (chunks + 3) / 4;
+  const int row = row0 + r;
+  const T* x_row = x + (size_t)(row < n ? row : 0) * ldx + (size_t)b * Ni;
+  f32x4 acc[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int st = 0; st < steps; ++st) {
+    const int chunk = st * 4 + g;
+    const bool in = chunk < chunks;
+    const Frag xf = (in && row < n) ? tw_load_frag(x_row + chunk * EPF) : Elem<T>::zero();
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const int o = cg * 64 + t * 16 + r;
+      const Frag wf = (in && o < No) ? tw_load_frag(w + ((size_t)b * No + o) * Ni + chunk * EPF) : Elem<T>::zero();
+      tw_mma16(acc[t], wf, xf);                            // D[output 4g + e][row r]
+    }
+  }
+  if (row >= n) return;
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    const int o = cg * 64 + t * 16 + 4 * g;
+    if (o < No) {
+      f32x4 v = acc[t];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] += bias ? bias[(size_t)b * No + o + e] : 0.f;
+      *reinterpret_cast<f32x4*>(out + (size_t)row * ldo + (size_t)b * No + o) = v;
+    }
+  }
+}
+
+extern "C" int tw_block_diagonal(int dtype, const void* x, long ldx, const void* w, const float* bias, float* out,
+                                 long ldo, int n, int blocks, int Ni, int No, hipStream_t stream) {
+  const int epf = dtype == TW_DTYPE_BF16 ? 8 : 4;
+  TW_REQUIRE(x && w && out && n >= 0 && blocks > 0 && Ni > 0 && No > 0);
+  TW_REQUIRE(dtype == TW_DTYPE_BF16 || dtype == TW_DTYPE_F32);
+  TW_REQUIRE(Ni % epf == 0 && No % 16 == 0 && ldx % epf == 0 && ldx >= (long)blocks * Ni && ldo % 4 == 0 && ldo >= (long)blocks * No);
+  TW_REQUIRE((uintptr_t)x % 16 == 0 && (uintptr_t)w % 16 == 0 && (uintptr_t)out % 16 == 0);
+  if (n == 0) return 0;
+  const int col_groups = tw_div_up(No, 64);
+  const dim3 grid(tw_div_up((long)blocks * col_groups, 4), tw_div_up(n, 16));
+  if (dtype == TW_DTYPE_BF16)
+    block_diagonal_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w, bias, out, ldo, n, blocks, Ni, No, col_groups);
+  else
+    block_diagonal_kernel<float><<<grid, 256, 0, stream>>>((const float*)x, ldx, (const float*)w, bias, out, ldo, n, blocks, Ni, No, col_groups);
   return TW_LAUNCH_RESULT();
 }
 
@@ -309,13 +454,21 @@ __global__ __launch_bounds__(256) void layer_end_kernel(float* __restrict__ x, c
     sum = tw_block_sum(sum, red);
     scale = mult * rsqrtf(sum / (float)width + eps);
   }
-  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+  const int share = (width + gridDim.y - 1) / gridDim.y;
+  const int c_end = min(width, (int)(blockIdx.y + 1) * share);
+  for (int c = blockIdx.y * share + threadIdx.x; c < c_end; c += blockDim.x) {
     float v = x[row + c];
     if (y) v += scale * y[row + c] * w[c];
     if (history) history[(size_t)(layer + 1) * history_stride + row + c] = v;
     if (mix) {
       float acc = mix[layer + 1] * v;
-      for (int j = 0; j <= layer; ++j) acc += mix[j] * history[(size_t)j * history_stride + row + c];
+      int j = 0;
+      for (; j + 4 <= layer + 1; j += 4) {
+        const float h0 = history[(size_t)j * history_stride + row + c], h1 = history[(size_t)(j + 1) * history_stride + row + c];
+        const float h2 = history[(size_t)(j + 2) * history_stride + row + c], h3 = history[(size_t)(j + 3) * history_stride + row + c];
+        acc += mix[j] * h0 + mix[j + 1] * h1 + mix[j + 2] * h2 + mix[j + 3] * h3;
+      }
+      for (; j <= layer; ++j) acc += mix[j] * history[(size_t)j * history_stride + row + c];
       v = acc;
     }
     x[row + c] = v;
@@ -327,6 +480,8 @@ extern "C" int tw_layer_end(float* x, const float* y, const float* w, float eps,
   TW_REQUIRE(x && n >= 0 && width > 0 && layer >= 0 && (!y || w) && (!mix || history));
   TW_REQUIRE(!history || history_stride >= (long)n * width);
   if (n == 0) return 0;
-  layer_end_kernel<<<n, 256, 0, stream>>>(x, y, w, eps, mult, history, history_stride, layer, mix, width);
+  int shares = n >= 512 ? 1 : tw_div_up(width, 512);
+  if (shares > 8) shares = 8;
+  layer_end_kernel<<<dim3(n, shares), 256, 0, stream>>>(x, y, w, eps, mult, history, history_stride, layer, mix, width);
   return TW_LAUNCH_RESULT();
 }

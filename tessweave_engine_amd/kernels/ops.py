@@ -518,25 +518,62 @@ def causal_conv(src, taps, state, q_start, kv_len, state_slots, phase, n_seqs, o
           "causal_conv")
 
 
-def gated_recurrence(gates, u, branch, lam, state, q_start, state_slots, n_seqs, out, blocks, decay, out_scale=1.0):
+def gated_recurrence_workspace_floats(n_seqs, max_q_len, channels):
+    return int(library().tw_gated_recurrence_workspace_floats(int(n_seqs), int(max_q_len), int(channels)))
+
+
+def gated_recurrence(gates, u, branch, lam, state, q_start, state_slots, n_seqs, max_q_len, out, blocks, decay,
+                     out_scale=1.0, out_pad=0, workspace=None):
     """The gated linear recurrence S = a S + sqrt(1 - a^2) i u per sequence and channel, a = exp(-decay *
     sigmoid(gate_a) * softplus(lam)); out = out_scale * S * gelu_tanh(branch). gates float32 [n, 2C], block b's
     recurrence gates at columns [2 b C/blocks, ...) followed by its input gates; u float32 [n, C]; branch and
-    out have the compute type; state float32 [requests, C]."""
+    out have the compute type; state float32 [requests, C]. max_q_len: the longest portion of the step; portions
+    longer than a chunk are walked by several threads a channel and need a float32 workspace
+    (`gated_recurrence_workspace_floats`). out_pad: further columns of out that are set to zero."""
     n, C, ld_u = _rows(u, "u")
     ng, cg, ld_g = _rows(gates, "gates")
     nb, cb, ld_b = _rows(branch, "branch")
     no, co, ld_o = _rows(out, "out")
     _need(gates.dtype == torch.float32 and u.dtype == torch.float32, "gates and u must be float32")
-    _need((ng, cg) == (n, 2 * C) and (nb, cb) == (n, C) and (no, co) == (n, C) and branch.dtype == out.dtype,
+    _need((ng, cg) == (n, 2 * C) and (nb, cb) == (n, C) and (no, co) == (n, C + out_pad) and branch.dtype == out.dtype,
           "gated_recurrence shapes do not agree")
     _need(C % blocks == 0 and lam.numel() == C and lam.dtype == torch.float32, "lam must be float32 [C], C a multiple of blocks")
     _need(state.dtype == torch.float32 and state.is_contiguous() and state.shape[-1] == C and state.dim() == 2,
           "state must be float32 [requests, C]")
+    _need(q_start.numel() >= n_seqs + 1 and state_slots.numel() >= n_seqs and 1 <= max_q_len, "sequence metadata is too short")
+    need = gated_recurrence_workspace_floats(n_seqs, max_q_len, C)
+    if need:
+        _need(workspace is not None and workspace.dtype == torch.float32 and workspace.numel() >= need,
+              "portions longer than a chunk need a float32 workspace")
     check(library().tw_gated_recurrence(dtype_id(out.dtype), _dev(gates), ld_g, _dev(u), ld_u, _dev(branch), ld_b,
                                         _dev(lam), _dev(state), _dev(q_start, torch.int32, "q_start"),
-                                        _dev(state_slots, torch.int32, "state_slots"), _dev(out), ld_o, int(n_seqs), C,
-                                        int(blocks), float(decay), float(out_scale), _stream()), "gated_recurrence")
+                                        _dev(state_slots, torch.int32, "state_slots"), _dev(out), ld_o, int(n_seqs),
+                                        int(max_q_len), C, int(blocks), int(out_pad), float(decay), float(out_scale),
+                                        _dev(workspace) if need else None, workspace.numel() if need else 0, _stream()),
+          "gated_recurrence")
+    return out
+
+
+def can_block_diagonal(x, weight):
+    """Does `block_diagonal` take these operands? (blocks of a multiple of 16 bytes in, a multiple of 16 out, aligned rows)"""
+    epf = 16 // x.element_size()
+    blocks, n_out, n_in = weight.shape
+    return (n_in % epf == 0 and n_out % 16 == 0 and x.stride(0) % epf == 0 and x.data_ptr() % 16 == 0
+            and x.shape[1] == blocks * n_in)
+
+
+def block_diagonal(x, weight, bias, out):
+    """out[n, b * No + o] = sum_i x[n, b * Ni + i] * weight[b, o, i] + bias[b * No + o]; weight [blocks, No, Ni] of x's
+    type, out float32 [n, blocks * No]."""
+    n, width, ldx = _rows(x, "x")
+    blocks, n_out, n_in = weight.shape
+    no, wo, ldo = _rows(out, "out")
+    _need(weight.is_contiguous() and weight.dtype == x.dtype and can_block_diagonal(x, weight), "block_diagonal: unsupported operands")
+    _need(out.dtype == torch.float32 and (no, wo) == (n, blocks * n_out) and ldo % 4 == 0 and out.data_ptr() % 16 == 0,
+          "out must be float32 [n, blocks * No] with 16-byte aligned rows")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.is_contiguous() and bias.numel() == blocks * n_out), "bias has the wrong size")
+    check(library().tw_block_diagonal(dtype_id(x.dtype), _dev(x), ldx, _dev(weight), _dev(bias) if bias is not None else None,
+                                      _dev(out), ldo, n, blocks, n_in, n_out, _stream()), "block_diagonal")
     return out
 
 

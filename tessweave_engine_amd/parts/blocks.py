@@ -8,7 +8,7 @@ import torch
 
 from ..cache.spec import CacheNeed
 from ..kernels import ops
-from ..weights.spec import NORMAL, VECTOR, TensorSpec
+from ..weights.spec import AVERAGE, VECTOR, TensorSpec
 from .base import Block, fold_pending
 
 
@@ -72,7 +72,7 @@ class DepthMixedBlock(Block):
     def tensor_specs(self):
         specs = [s for p in self.parts() for s in p.tensor_specs()]
         if self.mix_name:
-            specs.append(TensorSpec(self.mix_name, (self.layer + 2,), VECTOR, NORMAL))
+            specs.append(TensorSpec(self.mix_name, (self.layer + 2,), VECTOR, AVERAGE))
         return specs
 
     def bind(self, tensors, dtype, device):

@@ -20,7 +20,7 @@ import torch
 
 from ..cache.spec import CacheNeed, FixedState, PagedKV
 from ..kernels import ops
-from ..weights.spec import MATRIX, NORMAL, VECTOR, TensorSpec
+from ..weights.spec import IDENTITY_PLUS_NORMAL, MATRIX, NORMAL, VECTOR, TensorSpec
 from .base import Mixer, Part
 from .convolution import CausalConv
 from .linear import JoinedLinear, Linear
@@ -90,7 +90,7 @@ class MixedHeadAttention(MixerBranch):
     def tensor_specs(self):
         specs = []
         if self.has_talk:
-            specs.append(TensorSpec(self._name(4), (self.q_heads, self.q_heads), VECTOR, NORMAL))
+            specs.append(TensorSpec(self._name(4), (self.q_heads, self.q_heads), VECTOR, IDENTITY_PLUS_NORMAL))
         if self.has_sink:
             specs.append(TensorSpec(self._name(5), (self.q_heads,), VECTOR, NORMAL))
         return specs
@@ -177,7 +177,13 @@ class GatedLinearRecurrence(MixerBranch):
         ra, ri = tensors.pop(self._name(3)), tensors.pop(self._name(4))
         ra_b, ri_b = tensors.pop(self._name(3) + self.bias_suffix), tensors.pop(self._name(4) + self.bias_suffix)
         self.gates = []
-        for b in range(self.blocks):
+        # [blocks, 2n, n]: a block's recurrence gate rows, then its input gate rows; one kernel for all blocks
+        # where the sizes allow it, else one product a block
+        self.gate_weight = torch.cat([ra, ri], 1).contiguous()
+        self.gate_bias = torch.cat([ra_b, ri_b], 1).contiguous().view(-1)
+        probe = torch.empty(1, self.width_dev, dtype=self.gate_weight.dtype, device=self.gate_weight.device)[:, :self.width]
+        self.gates_fused = torch.device(device).type == "cuda" and ops.can_block_diagonal(probe, self.gate_weight)
+        for b in range(0 if not self.gates_fused else self.blocks, self.blocks):
             # the recurrence gate and the input gate of a block read the same inputs: one product for both
             name = f"{self.prefix}gates.{b}"
             gate = Linear([name], n, [2 * n], bias=True)
@@ -187,7 +193,7 @@ class GatedLinearRecurrence(MixerBranch):
         self.lam = tensors.pop(self._name(5)).contiguous()
 
     def weight_tensors(self):
-        return [self.lam]
+        return [self.lam] + ([self.gate_weight, self.gate_bias] if self.gates_fused else [])
 
     def cache_need(self):
         return CacheNeed(states=(self.conv.state_need(), (self.state_prefix + ".s", FixedState((self.width,), "float32"))))
@@ -200,13 +206,19 @@ class GatedLinearRecurrence(MixerBranch):
         self.conv.forward(ctx, run, linear, out=u, out32=u32)
         gates = ctx.scratch("recurrent.gates", (n, 2 * R), torch.float32)
         bs = R // self.blocks
+        if self.gates_fused:
+            ops.block_diagonal(u, self.gate_weight, self.gate_bias, gates)
         for b, gate in enumerate(self.gates):
             gate.forward(ctx, u[:, b * bs:(b + 1) * bs], gates[:, 2 * b * bs:2 * (b + 1) * bs])
         state = ctx.cache.states[run.cache_slot][self.state_prefix + ".s"]
-        ops.gated_recurrence(gates, u32, branch, self.lam, state, ctx.q_start, ctx.state_slots, ctx.n_seqs,
-                             out[:, :R], self.blocks, self.decay, out_scale=scale)
-        if self.width_dev > R:
-            out[:, R:].zero_()            # the tail meets zero columns of the output matrix, but must not hold NaN
+        longest = max(ctx.max_q_len, 1)
+        ws = None
+        floats = ops.gated_recurrence_workspace_floats(ctx.n_seqs, longest, R)
+        if floats:
+            ws = ctx.workspace.get("recurrent.chunks", (floats,), torch.float32)
+        # (the columns beyond R meet zero columns of the output matrix, but must not hold NaN: the kernel clears them)
+        ops.gated_recurrence(gates, u32, branch, self.lam, state, ctx.q_start, ctx.state_slots, ctx.n_seqs, longest,
+                             out, self.blocks, self.decay, out_scale=scale, out_pad=self.width_dev - R, workspace=ws)
 
 
 class ParallelMixer(Mixer):

@@ -4,7 +4,8 @@ The reference has no such mode; its tests draw random weights by building a
 library model under a fixed seed (tests/test_engine.py:15-25). Here every tensor
 is drawn by NAME: its generator is seeded from (seed, tensor name), so a
 tensor's values do not depend on which other tensors exist or on their order.
-Linear, embedding and bias values are N(0, std); norm weights are 1 + N(0, std).
+Linear, embedding and bias values are N(0, std); norm weights are 1 + N(0, std); the weights of an average
+over earlier results are (1 + N(0, std)) / entries; a matrix that mixes heads is the identity + N(0, std).
 """
 from __future__ import annotations
 
@@ -14,7 +15,7 @@ from pathlib import Path
 
 import torch
 
-from .spec import ONE_PLUS_NORMAL, TABLE
+from .spec import AVERAGE, IDENTITY_PLUS_NORMAL, ONE_PLUS_NORMAL, TABLE
 from .loader import device_dtype_for, resolve_dtype
 
 DEFAULT_STD = 0.02
@@ -34,6 +35,10 @@ def draw_tensor(spec, seed, std=DEFAULT_STD, device="cpu", dtype=torch.float32):
     t.normal_(0.0, std, generator=generator)
     if spec.init == ONE_PLUS_NORMAL:
         t += 1.0
+    elif spec.init == AVERAGE:
+        t = (t + 1.0) / max(1, t.numel())
+    elif spec.init == IDENTITY_PLUS_NORMAL:
+        t += torch.eye(spec.shape[0], spec.shape[1], device=device)
     return t.to(dtype)
 
 

@@ -12,6 +12,8 @@ MATRIX, VECTOR, TABLE = "matrix", "vector", "table"
 
 # Initialisations of the random-weights mode.
 NORMAL, ONE_PLUS_NORMAL = "normal", "one_plus_normal"
+# weights of an average over the tensor's entries: (1 + N(0, std)) / entries; a square matrix near the identity
+AVERAGE, IDENTITY_PLUS_NORMAL = "average", "identity_plus_normal"
 
 
 @dataclass(frozen=True)

@@ -91,9 +91,9 @@ def gated_recurrence(u, gate_a, gate_i, lam, state=None):
 
 def block_diagonal(u, weight, bias):
     """u [T, R] in `blocks` equal parts, part b times weight[b] ([out, in]) plus bias[b]."""
-    B, n, _ = weight.shape
-    parts = u.view(u.shape[0], B, n)
-    return (torch.einsum("tbi,boi->tbo", parts, weight) + bias).reshape(u.shape[0], B * n)
+    B, n_out, n_in = weight.shape
+    parts = u.view(u.shape[0], B, n_in)
+    return (torch.einsum("tbi,boi->tbo", parts, weight) + bias).reshape(u.shape[0], B * n_out)
 
 
 def recurrent_branch(h, w, p):

@@ -165,7 +165,7 @@ def test_causal_conv_over_portions_and_reused_slots(device, dtype, taps, norm):
 def test_gated_recurrence_carries_its_state(device, dtype):
     from tessweave_engine_amd.kernels import ops
     g = torch.Generator().manual_seed(5)
-    R, blocks, T, dt = 24, 3, 40, tdtype(dtype)
+    R, blocks, T, dt = 24, 3, 400, tdtype(dtype)
     bs = R // blocks
     u = torch.randn(T, R, generator=g)
     ga, gi = torch.randn(T, R, generator=g) * 2, torch.randn(T, R, generator=g) * 2
@@ -178,17 +178,41 @@ def test_gated_recurrence_carries_its_state(device, dtype):
     state = torch.zeros(2, R, device=device)
     state[0] = float("nan")                                # another request's slot
     got, at = [], 0
-    for n in (1, 5, 2, 1, 17, 14):
-        out = torch.empty(n, R, dtype=dt, device=device)
+    for n in (1, 5, 2, 1, 17, 14, 64, 65, 200, 31):          # portions of one chunk, of exactly one, and of several
+        out = torch.full((n, R + 3), float("nan"), dtype=dt, device=device)
+        floats = ops.gated_recurrence_workspace_floats(1, n, R)
+        assert (floats > 0) == (n > 64)
+        ws = torch.full((max(floats, 1),), float("nan"), device=device)
         ops.gated_recurrence(gates[at:at + n].contiguous().to(device), u[at:at + n].contiguous().to(device),
                              branch[at:at + n].to(dt).to(device), lam.to(device), state,
                              torch.tensor([0, n], dtype=torch.int32, device=device),
-                             torch.tensor([1], dtype=torch.int32, device=device), 1, out, blocks, 8.0, out_scale=0.7)
-        got.append(out.float().cpu())
+                             torch.tensor([1], dtype=torch.int32, device=device), 1, n, out, blocks, 8.0, out_scale=0.7,
+                             out_pad=3, workspace=ws)
+        assert (out[:, R:] == 0).all()
+        got.append(out[:, :R].float().cpu())
         at += n
     tol = 1e-5 if dtype == "float32" else 1e-2
     assert torch.allclose(torch.cat(got).double(), want, atol=tol, rtol=tol)
     assert torch.allclose(state[1].cpu().double(), S[-1], atol=1e-5, rtol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("n,blocks,n_in,n_out", [(1, 3, 8, 16), (37, 2, 40, 80), (130, 16, 128, 256)])
+def test_block_diagonal_product(device, dtype, n, blocks, n_in, n_out):
+    from tessweave_engine_amd.kernels import ops
+    g = torch.Generator().manual_seed(n)
+    dt = tdtype(dtype)
+    x = torch.randn(n, blocks * n_in, generator=g).to(dt)
+    w = (torch.randn(blocks, n_out, n_in, generator=g) / math.sqrt(n_in)).to(dt)
+    bias = torch.randn(blocks * n_out, generator=g)
+    want = plain.block_diagonal(x.double(), w.double(), bias.double().view(blocks, n_out))
+    wide = torch.zeros(n, blocks * n_in + 8, dtype=dt, device=device)          # rows further apart than they are long
+    wide[:, :blocks * n_in] = x.to(device)
+    out = torch.empty(n, blocks * n_out, device=device)
+    assert ops.can_block_diagonal(wide[:, :blocks * n_in], w.to(device))
+    ops.block_diagonal(wide[:, :blocks * n_in], w.to(device), bias.to(device), out)
+    tol = 2e-5 if dtype == "float32" else 2e-2
+    assert torch.allclose(out.cpu().double(), want, atol=tol, rtol=tol)
 
 
 def test_small_kernels(device):
