@@ -45,21 +45,24 @@ struct MixedAttnArgs {
   float* part;                       // splits > 1: [seq - seq0][split][H][E + 2] (output sums, max, sum)
   float scale, out_scale;
   int H, G, D, E, P, window, splits;
+  int q_in_lds;                      // 0: the tile's queries do not fit LDS beside the raw scores; fragments are read from memory
 };
 
-// Dynamic LDS: q tile [H][16][D + pad] of T, raw scores [2][H][64] of f32x4, talk [H][H] floats.
+// Dynamic LDS: q tile [H][16][D + pad] of T (if it fits), raw scores [2][H][64] of f32x4, talk [H][H] floats.
 template <typename T>
 __host__ __device__ inline size_t mx_q_row(int D) { return (size_t)D + 16 / sizeof(T); }
 
 template <typename T>
-static size_t mx_lds_bytes(int H, int D) {
-  size_t q = (size_t)H * 16 * mx_q_row<T>(D) * sizeof(T);
+static size_t mx_lds_bytes(int H, int D, bool q_in_lds) {
+  size_t q = q_in_lds ? (size_t)H * 16 * mx_q_row<T>(D) * sizeof(T) : 0;
   q = (q + 15) / 16 * 16;
   return q + (size_t)2 * H * 64 * 16 + (size_t)H * H * 4;
 }
 
-template <typename T, int HPW, int VT>
-__global__ __launch_bounds__(1024) void attn_mixed_kernel(MixedAttnArgs a) {
+// HPW heads a wave, VT 16-column tiles of a head's values, WMAX the most waves a workgroup may have (it sets the
+// registers a lane may use), AHEAD whether key fragments are requested a tile ahead (it costs registers).
+template <typename T, int HPW, int VT, int WMAX, bool AHEAD>
+__global__ __launch_bounds__(WMAX * 64) void attn_mixed_kernel(MixedAttnArgs a) {
   typedef typename Elem<T>::Frag Frag;
   typedef typename MxQuad<T>::Type Quad;
   constexpr int EPF = Elem<T>::kPerFrag;
@@ -67,7 +70,7 @@ __global__ __launch_bounds__(1024) void attn_mixed_kernel(MixedAttnArgs a) {
   const int H = a.H, D = a.D, E = a.E, P = a.P;
   const size_t qrow = mx_q_row<T>(D);
   T* lds_q = (T*)lds_raw;
-  size_t q_bytes = (size_t)H * 16 * qrow * sizeof(T);
+  size_t q_bytes = a.q_in_lds ? (size_t)H * 16 * qrow * sizeof(T) : 0;
   q_bytes = (q_bytes + 15) / 16 * 16;
   f32x4* lds_s = (f32x4*)(lds_raw + q_bytes);
   float* lds_talk = (float*)(lds_raw + q_bytes + (size_t)2 * H * 64 * 16);
@@ -87,7 +90,7 @@ __global__ __launch_bounds__(1024) void attn_mixed_kernel(MixedAttnArgs a) {
   const int chunks = D / EPF, steps = (chunks + 3) / 4, dts = E / 16;
 
   // ---- stage the tile's queries and the mixing matrix ------------------------------------------------
-  for (int i = threadIdx.x; i < H * 16 * chunks; i += blockDim.x) {
+  for (int i = threadIdx.x; i < (a.q_in_lds ? H * 16 * chunks : 0); i += blockDim.x) {
     const int chunk = i % chunks, row = (i / chunks) % 16, head = i / (chunks * 16);
     Frag f = Elem<T>::zero();
     if (row < n_rows)
@@ -123,40 +126,101 @@ __global__ __launch_bounds__(1024) void attn_mixed_kernel(MixedAttnArgs a) {
   }
   const T* keys = (const T*)a.keys;
   const T* values = (const T*)a.values;
+  const T* q_global = (const T*)a.q + (size_t)(q0 + tile * 16 + (r < n_rows ? r : 0)) * a.ldq;
+  auto q_frag = [&](int head, int chunk) -> Frag {
+    if (chunk >= chunks) return Elem<T>::zero();
+    if (a.q_in_lds) return *reinterpret_cast<const Frag*>(lds_q + ((size_t)head * 16 + r) * qrow + chunk * EPF);
+    return r < n_rows ? tw_load_frag(q_global + (size_t)head * D + chunk * EPF) : Elem<T>::zero();
+  };
+  // The K fragments of a key tile are requested one tile ahead (while the tile before is mixed and multiplied
+  // with its values), the V quads of a tile before the barrier that publishes its raw scores: a tile then waits
+  // for memory once, not twice, and mostly not at all. KP fragments a head fit the registers kept for that
+  // (head sizes up to 128 in bfloat16, 64 in float32); longer heads load their fragments where they are used.
+  constexpr int KP = AHEAD ? 4 : 1;
+  const bool ahead = AHEAD && steps <= KP;
+  Frag kpre[HPW][KP];
+  auto request_keys = [&](int kt) {
+    if constexpr (!AHEAD) return;
+    const int p = kt * 16 + r;
+    int page = -1;
+    if (kt < tile_hi && p < kv_len && p >= lo) page = table[p / P];
+#pragma unroll
+    for (int i = 0; i < HPW; ++i) {
+      const int head = wave * HPW + i;
+      const int kvh = (head < H ? head : 0) / heads_per_kv;
+      const T* k_row = keys + (((size_t)(page < 0 ? 0 : page) * a.G + kvh) * P + p % P) * D;
+#pragma unroll
+      for (int st = 0; st < KP; ++st) {
+        const int chunk = st * 4 + g;
+        kpre[i][st] = (page >= 0 && head < H && chunk < chunks) ? tw_load_frag(k_row + chunk * EPF) : Elem<T>::zero();
+      }
+    }
+  };
+  if (ahead) request_keys(tile_lo);
   int buf = 0;
   for (int kt = tile_lo; kt < tile_hi; ++kt, buf ^= 1) {
     const int p0 = kt * 16;
     // ---- raw scores of this wave's heads ---------------------------------------------------------------
+    f32x4 raw_own[HPW];
     {
       const int p = p0 + r;
       int page = -1;
-      if (p < kv_len && p >= lo) page = table[p / P];
+      if (!ahead && p < kv_len && p >= lo) page = table[p / P];
 #pragma unroll
       for (int i = 0; i < HPW; ++i) {
         const int head = wave * HPW + i;
+        raw_own[i] = f32x4{0.f, 0.f, 0.f, 0.f};
         if (head < H) {
-          const int kvh = head / heads_per_kv;
-          const T* k_row = keys + (((size_t)(page < 0 ? 0 : page) * a.G + kvh) * P + p % P) * D;
-          const T* q_row = lds_q + ((size_t)head * 16 + r) * qrow;
           f32x4 s = {0.f, 0.f, 0.f, 0.f};
-          for (int st = 0; st < steps; ++st) {
-            const int chunk = st * 4 + g;
-            const bool in = chunk < chunks;
-            const Frag kf = (page >= 0 && in) ? tw_load_frag(k_row + chunk * EPF) : Elem<T>::zero();
-            const Frag qf = in ? *reinterpret_cast<const Frag*>(q_row + chunk * EPF) : Elem<T>::zero();
-            tw_mma16(s, kf, qf);
+          if (AHEAD && ahead) {
+#pragma unroll
+            for (int st = 0; st < KP; ++st) {
+              const int chunk = st * 4 + g;
+              if (st < steps) {
+                tw_mma16(s, kpre[i][st], q_frag(head, chunk));
+              }
+            }
+          } else {
+            const int kvh = head / heads_per_kv;
+            const T* k_row = keys + (((size_t)(page < 0 ? 0 : page) * a.G + kvh) * P + p % P) * D;
+            for (int st = 0; st < steps; ++st) {
+              const int chunk = st * 4 + g;
+              const bool in = chunk < chunks;
+              const Frag kf = (page >= 0 && in) ? tw_load_frag(k_row + chunk * EPF) : Elem<T>::zero();
+              tw_mma16(s, kf, q_frag(head, chunk));
+            }
           }
 #pragma unroll
           for (int e = 0; e < 4; ++e) s[e] = s[e] * a.scale - slope[i] * (float)(t_row - (p0 + 4 * g + e));
-          lds_s[((size_t)buf * H + head) * 64 + lane] = s;
+          raw_own[i] = s;
         }
       }
     }
-    __syncthreads();
-    // ---- mix, mask, online softmax, O^T += V^T P^T ------------------------------------------------------------
+    // ---- this tile's values, then the next tile's keys: both are on their way during the mixing -----------------
     const int pv = p0 + 4 * g;
     int vpage = -1;
     if (pv < kv_len && pv + 3 >= lo) vpage = table[pv / P];
+    Quad vq[HPW][VT];
+#pragma unroll
+    for (int i = 0; i < HPW; ++i) {
+      const int head = wave * HPW + i;
+      const int kvh = (head < H ? head : 0) / heads_per_kv;
+      const T* v_base = values + ((size_t)(vpage < 0 ? 0 : vpage) * a.G + kvh) * E * P + pv % P;
+#pragma unroll
+      for (int dt = 0; dt < VT; ++dt) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) vq[i][dt][e] = tw_from_float<T>(0.f);
+        if (dt < dts && vpage >= 0 && head < H) vq[i][dt] = *reinterpret_cast<const Quad*>(v_base + (size_t)(dt * 16 + r) * P);
+      }
+    }
+    if (ahead) request_keys(kt + 1);
+#pragma unroll
+    for (int i = 0; i < HPW; ++i) {
+      const int head = wave * HPW + i;
+      if (head < H) lds_s[((size_t)buf * H + head) * 64 + lane] = raw_own[i];
+    }
+    __syncthreads();
+    // ---- mix, mask, online softmax, O^T += V^T P^T ------------------------------------------------------------
 #pragma unroll
     for (int i = 0; i < HPW; ++i) {
       const int head = wave * HPW + i;
@@ -191,24 +255,16 @@ __global__ __launch_bounds__(1024) void attn_mixed_kernel(MixedAttnArgs a) {
         sum = tw_rows_sum(sum);
         l[i] = l[i] * alpha + sum;
         m[i] = m_new;
-        const int kvh = head / heads_per_kv;
-        const T* v_base = values + ((size_t)(vpage < 0 ? 0 : vpage) * a.G + kvh) * E * P + pv % P;
 #pragma unroll
         for (int dt = 0; dt < VT; ++dt) {
           if (dt < dts) {
-            Quad vq;
-            if (vpage >= 0) {
-              vq = *reinterpret_cast<const Quad*>(v_base + (size_t)(dt * 16 + r) * P);
+            Quad v = vq[i][dt];
 #pragma unroll
-              for (int e = 0; e < 4; ++e)
-                if (pv + e >= kv_len || pv + e < lo) vq[e] = tw_from_float<T>(0.f);
-            } else {
-#pragma unroll
-              for (int e = 0; e < 4; ++e) vq[e] = tw_from_float<T>(0.f);
-            }
+            for (int e = 0; e < 4; ++e)
+              if (pv + e >= kv_len || pv + e < lo) v[e] = tw_from_float<T>(0.f);
 #pragma unroll
             for (int e = 0; e < 4; ++e) acc[i][dt][e] *= alpha;
-            tw_mma16_k4(acc[i][dt], vq, pr);
+            tw_mma16_k4(acc[i][dt], v, pr);
           }
         }
       }
@@ -264,9 +320,9 @@ __global__ void attn_mixed_merge_kernel(MixedAttnArgs a) {
   }
 }
 
-template <typename T, int HPW, int VT>
+template <typename T, int HPW, int VT, int WMAX, bool AHEAD>
 static int mixed_launch(const MixedAttnArgs& a, int n_seqs, int tiles, int waves, size_t lds, hipStream_t stream) {
-  auto kernel = attn_mixed_kernel<T, HPW, VT>;
+  auto kernel = attn_mixed_kernel<T, HPW, VT, WMAX, AHEAD>;
   if (lds > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
@@ -276,35 +332,39 @@ static int mixed_launch(const MixedAttnArgs& a, int n_seqs, int tiles, int waves
 }
 
 template <typename T>
-static int mixed_dispatch(const MixedAttnArgs& a, int n_seqs, int max_q_len, hipStream_t stream) {
+static int mixed_dispatch(const MixedAttnArgs& args, int n_seqs, int max_q_len, hipStream_t stream) {
   const int tiles = tw_div_up(max_q_len, 16);
   // One head a wave up to 16 heads; two a wave (values of up to 128 elements only: the output sums of a
   // wave's heads live in its registers) up to 32.
-  const int hpw = a.H <= 16 ? 1 : 2;
-  const int waves = tw_div_up(a.H, hpw);
-  const size_t lds = mx_lds_bytes<T>(a.H, a.D);
+  const int hpw = args.H <= 16 ? 1 : 2;
+  const int waves = tw_div_up(args.H, hpw);
+  MixedAttnArgs a = args;
+  a.q_in_lds = mx_lds_bytes<T>(a.H, a.D, true) <= 150 * 1024 ? 1 : 0;
+  const size_t lds = mx_lds_bytes<T>(a.H, a.D, a.q_in_lds != 0);
   TW_REQUIRE(waves <= 16 && lds <= 150 * 1024 && (hpw == 1 || a.E <= 128));
   int code;
   if (hpw == 2)
-    code = a.E <= 64 ? mixed_launch<T, 2, 4>(a, n_seqs, tiles, waves, lds, stream)
-                     : mixed_launch<T, 2, 8>(a, n_seqs, tiles, waves, lds, stream);
-  else if (a.E <= 64)
-    code = mixed_launch<T, 1, 4>(a, n_seqs, tiles, waves, lds, stream);
-  else if (a.E <= 128)
-    code = mixed_launch<T, 1, 8>(a, n_seqs, tiles, waves, lds, stream);
+    code = a.E <= 64 ? mixed_launch<T, 2, 4, 16, false>(a, n_seqs, tiles, waves, lds, stream)
+                     : mixed_launch<T, 2, 8, 16, false>(a, n_seqs, tiles, waves, lds, stream);
+  else if (waves <= 8)          // up to 8 heads: workgroups of up to 512 lanes, which may use twice the registers
+    code = a.E <= 64 ? mixed_launch<T, 1, 4, 8, true>(a, n_seqs, tiles, waves, lds, stream)
+         : a.E <= 128 ? mixed_launch<T, 1, 8, 8, true>(a, n_seqs, tiles, waves, lds, stream)
+                      : mixed_launch<T, 1, 16, 8, true>(a, n_seqs, tiles, waves, lds, stream);
   else
-    code = mixed_launch<T, 1, 16>(a, n_seqs, tiles, waves, lds, stream);
+    code = a.E <= 64 ? mixed_launch<T, 1, 4, 16, true>(a, n_seqs, tiles, waves, lds, stream)
+         : a.E <= 128 ? mixed_launch<T, 1, 8, 16, true>(a, n_seqs, tiles, waves, lds, stream)
+                      : mixed_launch<T, 1, 16, 16, false>(a, n_seqs, tiles, waves, lds, stream);
   if (code != 0 || a.splits == 1) return code;
   attn_mixed_merge_kernel<T><<<dim3(n_seqs, a.H), 64, 0, stream>>>(a);
   return TW_LAUNCH_RESULT();
 }
 
-// Key ranges for one-token sequences: enough workgroups to spread over the chip, each with at least 8 key tiles.
+// Key ranges for one-token sequences: enough workgroups to spread over the chip, each with at least 4 key tiles.
 extern "C" int tw_attn_mixed_splits(int n_seqs, int max_kv_len) {
   if (n_seqs <= 0) return 1;
   const int tiles = tw_div_up(max_kv_len, 16);
-  int want = 512 / n_seqs;
-  int most = tiles / 8;
+  int want = 1024 / n_seqs;
+  int most = tiles / 4;
   int s = want < most ? want : most;
   if (s > 64) s = 64;
   return s < 1 ? 1 : s;
@@ -335,7 +395,7 @@ extern "C" int tw_attn_mixed(int dtype, const void* q, long ldq, const void* key
   }
   if (n_seqs == 0) return 0;
   MixedAttnArgs a{q, ldq, keys, values, block_table, table_stride, q_start, kv_len, seq0, out, ldo, talk, sink, slopes,
-                  workspace, scale, out_scale, q_heads, kv_heads, key_dim, value_dim, page_size, window, splits};
+                  workspace, scale, out_scale, q_heads, kv_heads, key_dim, value_dim, page_size, window, splits, 1};
   if (dtype == TW_DTYPE_BF16) return mixed_dispatch<bf16_t>(a, n_seqs, max_q_len, stream);
   if (dtype == TW_DTYPE_F32) return mixed_dispatch<float>(a, n_seqs, max_q_len, stream);
   return TW_ERR_BAD_ARGUMENT;

@@ -55,6 +55,7 @@ def paged(keys, values, page, order):
     (4, 2, 32, 16, 9, 70, 70, 8),          # whole prompt, window crosses pages
     (3, 3, 16, 48, 0, 45, 13, 4),          # no window, a portion behind cached keys
     (20, 4, 16, 32, 33, 50, 50, 16),       # two heads a wave
+    (32, 8, 128, 64, 40, 90, 90, 16),      # so many long heads that a tile's queries stay in memory
     (2, 1, 80, 128, 17, 300, 1, 16),       # decode
     (6, 2, 64, 96, 0, 700, 1, 32),         # decode over many keys: several key ranges
 ])
@@ -91,7 +92,7 @@ def test_mixed_head_attention(device, dtype, H, G, D, E, window, T, q_len, page)
     splits, ws = 1, None
     if q_len == 1:
         splits = ops.attn_mixed_splits(1, T)
-        assert (splits > 1) == (T >= 256)
+        assert (splits > 1) == (T >= 128)
         ws = torch.empty(ops.attn_mixed_workspace_floats(1, H, E, splits), dtype=torch.float32, device=device)
     ops.attn_mixed(qd, kp, vp, table, q_start, kv_len, 0, 1, q_len, out, H, G, scale, window=window,
                    talk=talk.to(device), sink=sink.to(device), slopes=slopes, out_scale=0.5, splits=splits, workspace=ws)
