@@ -20,8 +20,9 @@
 // still in accumulator layout, are the B operand of O^T += V^T P^T. The raw-score buffer exists
 // twice, so one barrier per key tile is enough.
 //
-// Sequences with one token (decode) can have their keys cut into `splits` ranges for separate
-// workgroups; a second kernel merges the partial results in index order.
+// A tile's keys can be cut into `splits` ranges for separate workgroups (one-token sequences, whose only tile
+// would otherwise walk all keys alone; prompt portions with fewer tiles than the chip has CUs); a second kernel
+// merges the partial results in index order.
 #include "tw_common.h"
 
 template <typename T> __device__ __forceinline__ float mx_exp(float v);
@@ -42,9 +43,10 @@ struct MixedAttnArgs {
   const float* talk;                 // [H][H] or null
   const float* sink;                 // [H] or null
   const float* slopes;               // [H] or null
-  float* part;                       // splits > 1: [seq - seq0][split][H][E + 2] (output sums, max, sum)
+  float* part;                       // splits > 1: [seq - seq0][tile][split][H][rows_kept][E + 2] (output sums, max, sum)
   float scale, out_scale;
   int H, G, D, E, P, window, splits;
+  int rows_kept;                     // rows of a tile whose partial results are kept: 1 for one-token sequences, else 16
   int q_in_lds;                      // 0: the tile's queries do not fit LDS beside the raw scores; fragments are read from memory
 };
 
@@ -160,6 +162,9 @@ __global__ __launch_bounds__(WMAX * 64) void attn_mixed_kernel(MixedAttnArgs a) 
   int buf = 0;
   for (int kt = tile_lo; kt < tile_hi; ++kt, buf ^= 1) {
     const int p0 = kt * 16;
+    // A tile whose 16 keys every row of the query tile sees (none beyond the first row's position, none before
+    // the last row's window) needs no masks; most tiles of a long window are such.
+    const bool interior = p0 + 15 <= pos0 && (a.window == 0 || p0 >= pos0 + n_rows - a.window);
     // ---- raw scores of this wave's heads ---------------------------------------------------------------
     f32x4 raw_own[HPW];
     {
@@ -226,21 +231,34 @@ __global__ __launch_bounds__(WMAX * 64) void attn_mixed_kernel(MixedAttnArgs a) 
       const int head = wave * HPW + i;
       if (head < H) {
         f32x4 s = {0.f, 0.f, 0.f, 0.f};
-        for (int other = 0; other < H; ++other) {
-          const float w = lds_talk[head * H + other];
-          const f32x4 raw = lds_s[((size_t)buf * H + other) * 64 + lane];
+        const float* talk_row = lds_talk + head * H;
+        const f32x4* raw_lane = lds_s + (size_t)buf * H * 64 + lane;
+        int other = 0;
+        for (; other + 4 <= H; other += 4) {               // four heads' reads in flight at a time
+          const f32x4 r0 = raw_lane[(other + 0) * 64], r1 = raw_lane[(other + 1) * 64];
+          const f32x4 r2 = raw_lane[(other + 2) * 64], r3 = raw_lane[(other + 3) * 64];
+          const float w0 = talk_row[other], w1 = talk_row[other + 1], w2 = talk_row[other + 2], w3 = talk_row[other + 3];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) s[e] += w0 * r0[e] + w1 * r1[e] + w2 * r2[e] + w3 * r3[e];
+        }
+        for (; other < H; ++other) {
+          const float w = talk_row[other];
+          const f32x4 raw = raw_lane[other * 64];
 #pragma unroll
           for (int e = 0; e < 4; ++e) s[e] += w * raw[e];
         }
-        const int lo_row = a.window > 0 ? t_row - a.window + 1 : 0;
         float mx = -INFINITY;
+        if (!interior) {
+          const int lo_row = a.window > 0 ? t_row - a.window + 1 : 0;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int p = p0 + 4 * g + e;
-          const bool ok = p < kv_len && p <= t_row && p >= lo_row;
-          s[e] = ok ? s[e] : -INFINITY;
-          mx = fmaxf(mx, s[e]);
+          for (int e = 0; e < 4; ++e) {
+            const int p = p0 + 4 * g + e;
+            const bool ok = p < kv_len && p <= t_row && p >= lo_row;
+            s[e] = ok ? s[e] : -INFINITY;
+          }
         }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) mx = fmaxf(mx, s[e]);
         mx = tw_rows_max(mx);
         const float m_new = fmaxf(m[i], mx);
         const float m_use = m_new == -INFINITY ? 0.f : m_new;
@@ -255,15 +273,21 @@ __global__ __launch_bounds__(WMAX * 64) void attn_mixed_kernel(MixedAttnArgs a) 
         sum = tw_rows_sum(sum);
         l[i] = l[i] * alpha + sum;
         m[i] = m_new;
+        // the output sums are rescaled only when some row's maximum has moved (a branch the whole wave takes alike)
+        const bool rescale = __builtin_amdgcn_ballot_w64(alpha != 1.f) != 0;
 #pragma unroll
         for (int dt = 0; dt < VT; ++dt) {
           if (dt < dts) {
             Quad v = vq[i][dt];
+            if (!interior) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
-              if (pv + e >= kv_len || pv + e < lo) v[e] = tw_from_float<T>(0.f);
+              for (int e = 0; e < 4; ++e)
+                if (pv + e >= kv_len || pv + e < lo) v[e] = tw_from_float<T>(0.f);
+            }
+            if (rescale) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) acc[i][dt][e] *= alpha;
+              for (int e = 0; e < 4; ++e) acc[i][dt][e] *= alpha;
+            }
             tw_mma16_k4(acc[i][dt], v, pr);
           }
         }
@@ -284,8 +308,8 @@ __global__ __launch_bounds__(WMAX * 64) void attn_mixed_kernel(MixedAttnArgs a) 
         if (dt < dts)
 #pragma unroll
           for (int e = 0; e < 4; ++e) dst[dt * 16 + 4 * g + e] = tw_from_float<T>(acc[i][dt][e] * inv);
-    } else if (r == 0) {
-      float* dst = a.part + (((size_t)blockIdx.y * a.splits + blockIdx.z) * H + head) * (E + 2);
+    } else if (r < a.rows_kept) {
+      float* dst = a.part + (((((size_t)blockIdx.y * gridDim.x + tile) * a.splits + blockIdx.z) * H + head) * a.rows_kept + r) * (E + 2);
 #pragma unroll
       for (int dt = 0; dt < VT; ++dt)
         if (dt < dts)
@@ -299,24 +323,30 @@ __global__ __launch_bounds__(WMAX * 64) void attn_mixed_kernel(MixedAttnArgs a) 
   }
 }
 
-// Merge the partial results of a one-token sequence's key ranges, in index order. grid (n_seqs, H).
+// Merge the partial results of a tile's key ranges, in index order. grid (tiles, n_seqs, H).
 template <typename T>
-__global__ void attn_mixed_merge_kernel(MixedAttnArgs a) {
-  const int seq = a.seq0 + blockIdx.x, head = blockIdx.y;
-  const int token = a.q_start[seq];
+__global__ __launch_bounds__(256) void attn_mixed_merge_kernel(MixedAttnArgs a) {
+  const int seq = a.seq0 + blockIdx.y, head = blockIdx.z, tile = blockIdx.x;
+  const int q0 = a.q_start[seq], q_len = a.q_start[seq + 1] - q0;
+  if (tile * 16 >= q_len) return;
+  const int n_rows = min(min(16, q_len - tile * 16), a.rows_kept);
   const int E = a.E;
-  const float* base = a.part + ((size_t)blockIdx.x * a.splits * a.H + head) * (E + 2);
-  const size_t stride = (size_t)a.H * (E + 2);
-  float m = -INFINITY;
-  for (int s = 0; s < a.splits; ++s) m = fmaxf(m, base[s * stride + E]);
-  const float m_use = m == -INFINITY ? 0.f : m;
-  float l = 0.f;
-  for (int s = 0; s < a.splits; ++s) l += base[s * stride + E + 1] * mx_exp<T>(base[s * stride + E] - m_use);
-  const float inv = l > 0.f ? a.out_scale / l : 0.f;
-  for (int d = threadIdx.x; d < E; d += blockDim.x) {
-    float o = 0.f;
-    for (int s = 0; s < a.splits; ++s) o += base[s * stride + d] * mx_exp<T>(base[s * stride + E] - m_use);
-    ((T*)a.out)[(size_t)token * a.ldo + (size_t)head * E + d] = tw_from_float<T>(o * inv);
+  const size_t stride = (size_t)a.H * a.rows_kept * (E + 2);          // between key ranges
+  const float* tile_base = a.part + ((((size_t)blockIdx.y * gridDim.x + tile) * a.splits) * a.H + head) * a.rows_kept * (E + 2);
+  for (int i = threadIdx.x; i < n_rows * E; i += blockDim.x) {
+    const int row = i / E, d = i % E;
+    const float* base = tile_base + (size_t)row * (E + 2);
+    float m = -INFINITY;
+    for (int s = 0; s < a.splits; ++s) m = fmaxf(m, base[s * stride + E]);
+    const float m_use = m == -INFINITY ? 0.f : m;
+    float l = 0.f, o = 0.f;
+    for (int s = 0; s < a.splits; ++s) {
+      const float f = mx_exp<T>(base[s * stride + E] - m_use);
+      l += base[s * stride + E + 1] * f;
+      o += base[s * stride + d] * f;
+    }
+    const float inv = l > 0.f ? a.out_scale / l : 0.f;
+    ((T*)a.out)[(size_t)(q0 + tile * 16 + row) * a.ldo + (size_t)head * E + d] = tw_from_float<T>(o * inv);
   }
 }
 
@@ -340,6 +370,7 @@ static int mixed_dispatch(const MixedAttnArgs& args, int n_seqs, int max_q_len, 
   const int waves = tw_div_up(args.H, hpw);
   MixedAttnArgs a = args;
   a.q_in_lds = mx_lds_bytes<T>(a.H, a.D, true) <= 150 * 1024 ? 1 : 0;
+  a.rows_kept = max_q_len == 1 ? 1 : 16;
   const size_t lds = mx_lds_bytes<T>(a.H, a.D, a.q_in_lds != 0);
   TW_REQUIRE(waves <= 16 && lds <= 150 * 1024 && (hpw == 1 || a.E <= 128));
   int code;
@@ -355,7 +386,7 @@ static int mixed_dispatch(const MixedAttnArgs& args, int n_seqs, int max_q_len, 
          : a.E <= 128 ? mixed_launch<T, 1, 8, 16, true>(a, n_seqs, tiles, waves, lds, stream)
                       : mixed_launch<T, 1, 16, 16, false>(a, n_seqs, tiles, waves, lds, stream);
   if (code != 0 || a.splits == 1) return code;
-  attn_mixed_merge_kernel<T><<<dim3(n_seqs, a.H), 64, 0, stream>>>(a);
+  attn_mixed_merge_kernel<T><<<dim3(tiles, n_seqs, a.H), 256, 0, stream>>>(a);
   return TW_LAUNCH_RESULT();
 }
 
@@ -370,8 +401,20 @@ extern "C" int tw_attn_mixed_splits(int n_seqs, int max_kv_len) {
   return s < 1 ? 1 : s;
 }
 
-extern "C" long tw_attn_mixed_workspace_floats(int n_seqs, int q_heads, int value_dim, int splits) {
-  return (long)n_seqs * splits * q_heads * (value_dim + 2);
+// Key ranges for prompt portions: only where the row tiles alone would leave most of the chip idle and a tile
+// has keys enough to share out (each range at least 8 key tiles).
+extern "C" int tw_attn_mixed_prefill_splits(int n_tokens, int n_seqs, int max_kv_len) {
+  const int tiles = tw_div_up(n_tokens, 16) + n_seqs;
+  const int key_tiles = tw_div_up(max_kv_len, 16);
+  int s = 320 / (tiles > 0 ? tiles : 1);
+  if (s > key_tiles / 8) s = key_tiles / 8;
+  if (s > 8) s = 8;
+  return s < 1 ? 1 : s;
+}
+
+extern "C" long tw_attn_mixed_workspace_floats(int n_seqs, int max_q_len, int q_heads, int value_dim, int splits) {
+  const long tiles = tw_div_up(max_q_len, 16);
+  return (long)n_seqs * tiles * splits * q_heads * (max_q_len == 1 ? 1 : 16) * (value_dim + 2);
 }
 
 extern "C" int tw_attn_mixed(int dtype, const void* q, long ldq, const void* keys, const void* values,
@@ -390,12 +433,12 @@ extern "C" int tw_attn_mixed(int dtype, const void* q, long ldq, const void* key
   const int esize = dtype == TW_DTYPE_BF16 ? 2 : 4;
   TW_REQUIRE((ldq * esize) % 16 == 0);
   if (splits > 1) {
-    TW_REQUIRE(max_q_len == 1 && workspace != nullptr);
-    TW_REQUIRE(workspace_floats >= tw_attn_mixed_workspace_floats(n_seqs, q_heads, value_dim, splits));
+    TW_REQUIRE(workspace != nullptr);
+    TW_REQUIRE(workspace_floats >= tw_attn_mixed_workspace_floats(n_seqs, max_q_len, q_heads, value_dim, splits));
   }
   if (n_seqs == 0) return 0;
   MixedAttnArgs a{q, ldq, keys, values, block_table, table_stride, q_start, kv_len, seq0, out, ldo, talk, sink, slopes,
-                  workspace, scale, out_scale, q_heads, kv_heads, key_dim, value_dim, page_size, window, splits, 1};
+                  workspace, scale, out_scale, q_heads, kv_heads, key_dim, value_dim, page_size, window, splits, 16, 1};
   if (dtype == TW_DTYPE_BF16) return mixed_dispatch<bf16_t>(a, n_seqs, max_q_len, stream);
   if (dtype == TW_DTYPE_F32) return mixed_dispatch<float>(a, n_seqs, max_q_len, stream);
   return TW_ERR_BAD_ARGUMENT;

@@ -46,7 +46,8 @@ _SIGNATURES = {
     "tw_token_gate": (I, [I, P, P, L, P, P, I, I, I, P, I, I, P]),
     "tw_layer_end": (I, [P, P, P, F, F, P, L, I, P, I, I, P]),
     "tw_attn_mixed_splits": (I, [I, I]),
-    "tw_attn_mixed_workspace_floats": (L, [I, I, I, I]),
+    "tw_attn_mixed_prefill_splits": (I, [I, I, I]),
+    "tw_attn_mixed_workspace_floats": (L, [I, I, I, I, I]),
     "tw_attn_mixed": (I, [I, P, L, P, P, P, I, P, P, I, I, I, P, L, P, P, P, P, L, I, I, I, I, I, I, F, F, I, P]),
     "tw_kv_store": (I, [I, P, L, I, I, P, P, P, I, I, I, I, I, P]),
     "tw_sampling_uniform": (F, [c_uint64, c_uint64]),

@@ -638,8 +638,13 @@ def attn_mixed_splits(n_seqs, max_kv_len):
     return int(library().tw_attn_mixed_splits(int(n_seqs), int(max_kv_len)))
 
 
-def attn_mixed_workspace_floats(n_seqs, q_heads, value_dim, splits):
-    return int(library().tw_attn_mixed_workspace_floats(int(n_seqs), q_heads, value_dim, int(splits)))
+def attn_mixed_prefill_splits(n_tokens, n_seqs, max_kv_len):
+    """Key ranges for a launch over prompt portions (1: none): more than one only where there are few row tiles."""
+    return int(library().tw_attn_mixed_prefill_splits(int(n_tokens), int(n_seqs), int(max_kv_len)))
+
+
+def attn_mixed_workspace_floats(n_seqs, max_q_len, q_heads, value_dim, splits):
+    return int(library().tw_attn_mixed_workspace_floats(int(n_seqs), int(max_q_len), q_heads, value_dim, int(splits)))
 
 
 def kv_store(src, k_col, v_col, slots, keys, values, kv_heads, key_dim, value_dim):
@@ -663,7 +668,8 @@ def attn_mixed(q, keys, values, block_table, q_start, kv_len, seq0, n_seqs, max_
     q [rows, >= q_heads * key_dim] (head h at columns h * key_dim), keys [pages, kv_heads, page, key_dim], values
     [pages, kv_heads, value_dim, page], out [rows, q_heads * value_dim]. talk float32 [H, H] mixes the scores
     (None: no mixing), slopes float32 [H] take slope * distance off the raw scores, sink float32 [H] adds exp(sink)
-    to the softmax's denominator. splits > 1 (one-token sequences only) cuts the keys into ranges; needs a workspace.
+    to the softmax's denominator. splits > 1 cuts every tile's keys into ranges; needs a workspace
+    (`attn_mixed_workspace_floats`).
     """
     key_dim, value_dim, page = keys.shape[3], values.shape[2], keys.shape[2]
     nq, wq, ldq = _rows(q, "q")

@@ -126,13 +126,20 @@ class MixedHeadAttention(MixerBranch):
             ws = None
             if splits > 1:
                 # sized for the most splits any length class can ask for, so that it never grows under a capture
-                floats = ops.attn_mixed_workspace_floats(ctx.n_decode, H, E, max(splits, ops.attn_mixed_splits(ctx.n_decode, most)))
+                floats = ops.attn_mixed_workspace_floats(ctx.n_decode, 1, H, E, max(splits, ops.attn_mixed_splits(ctx.n_decode, most)))
                 ws = ctx.workspace.get("attn.mixed.split", (floats,), torch.float32)
             ops.attn_mixed(proj, keys, values, group.block_table, ctx.q_start, ctx.kv_len, 0, ctx.n_decode, 1, out,
                            H, G, self.scale, splits=splits, workspace=ws, **common)
         if ctx.n_seqs > ctx.n_decode:
+            n_seqs = ctx.n_seqs - ctx.n_decode
+            longest = min(ctx.max_kv_len, window + ctx.max_q_len) if window else ctx.max_kv_len
+            splits = ops.attn_mixed_prefill_splits(ctx.n_tokens - ctx.n_decode, n_seqs, longest)
+            ws = None
+            if splits > 1:
+                floats = ops.attn_mixed_workspace_floats(n_seqs, ctx.max_q_len, H, E, splits)
+                ws = ctx.workspace.get("attn.mixed.split.rows", (floats,), torch.float32)
             ops.attn_mixed(proj, keys, values, group.block_table, ctx.q_start, ctx.kv_len, ctx.n_decode,
-                           ctx.n_seqs - ctx.n_decode, ctx.max_q_len, out, H, G, self.scale, **common)
+                           n_seqs, ctx.max_q_len, out, H, G, self.scale, splits=splits, workspace=ws, **common)
 
 
 class GatedLinearRecurrence(MixerBranch):

@@ -58,6 +58,7 @@ def paged(keys, values, page, order):
     (32, 8, 128, 64, 40, 90, 90, 16),      # so many long heads that a tile's queries stay in memory
     (2, 1, 80, 128, 17, 300, 1, 16),       # decode
     (6, 2, 64, 96, 0, 700, 1, 32),         # decode over many keys: several key ranges
+    (5, 1, 32, 48, 200, 400, 150, 16),     # a portion whose tiles' keys are cut into ranges
 ])
 def test_mixed_head_attention(device, dtype, H, G, D, E, window, T, q_len, page):
     from tessweave_engine_amd.kernels import ops
@@ -93,7 +94,10 @@ def test_mixed_head_attention(device, dtype, H, G, D, E, window, T, q_len, page)
     if q_len == 1:
         splits = ops.attn_mixed_splits(1, T)
         assert (splits > 1) == (T >= 128)
-        ws = torch.empty(ops.attn_mixed_workspace_floats(1, H, E, splits), dtype=torch.float32, device=device)
+        ws = torch.empty(ops.attn_mixed_workspace_floats(1, 1, H, E, splits), dtype=torch.float32, device=device)
+    elif T >= 256:
+        splits = 3                                         # a prompt portion whose tiles' keys are cut into ranges
+        ws = torch.full((ops.attn_mixed_workspace_floats(1, q_len, H, E, splits),), float("nan"), device=device)
     ops.attn_mixed(qd, kp, vp, table, q_start, kv_len, 0, 1, q_len, out, H, G, scale, window=window,
                    talk=talk.to(device), sink=sink.to(device), slopes=slopes, out_scale=0.5, splits=splits, workspace=ws)
     got = out.float().cpu().numpy() / 0.5
