@@ -18,6 +18,7 @@ from __future__ import annotations
 import argparse
 from dataclasses import asdict
 import json
+import math
 from pathlib import Path
 import platform
 import sys
@@ -203,8 +204,14 @@ def main(argv=None):
                           "kv_fp32_bytes": layout.bytes_per_token(4) * tokens,
                           **formula,
                           "cache_groups": [{"layers": len(g.slots), "kv_heads": g.spec.kv_heads,
-                                            "head_dim": g.spec.head_dim, "window": g.spec.window}
+                                            "head_dim": g.spec.head_dim, "window": g.spec.window,
+                                            **({"value_dim": g.spec.value_dim} if g.spec.value_dim else {})}
                                            for g in layout.groups],
+                          # what a request holds besides pages: recurrent state, the last inputs of convolutions
+                          "state_bytes_per_request": sum(
+                              math.prod(spec.shape) * (2 if spec.dtype == "bfloat16" else 4)
+                              for need in layout.needs if need is not None
+                              for spec in ([need.state] if need.state else []) + [s for _, s in need.states]),
                           "excludes": ["weights", "activations and scratch buffers", "runtime/allocator"]}, indent=2))
     elif args.command == "replay":
         from .engine.trace import read_events

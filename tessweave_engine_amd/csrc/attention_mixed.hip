@@ -46,6 +46,7 @@ struct MixedAttnArgs {
   float* part;                       // splits > 1: [seq - seq0][tile][split][H][rows_kept][E + 2] (output sums, max, sum)
   float scale, out_scale;
   int H, G, D, E, P, window, splits;
+  int page_shift;                    // log2(P) if P is a power of two, else -1
   int rows_kept;                     // rows of a tile whose partial results are kept: 1 for one-token sequences, else 16
   int q_in_lds;                      // 0: the tile's queries do not fit LDS beside the raw scores; fragments are read from memory
 };
@@ -141,16 +142,26 @@ __global__ __launch_bounds__(WMAX * 64) void attn_mixed_kernel(MixedAttnArgs a) 
   constexpr int KP = AHEAD ? 4 : 1;
   const bool ahead = AHEAD && steps <= KP;
   Frag kpre[HPW][KP];
-  auto request_keys = [&](int kt) {
+  // Page numbers are looked up a tile before the loads that need them, so that no load waits for a lookup.
+  const int shift = a.page_shift;
+  auto page_of = [&](int p) { return shift >= 0 ? p >> shift : p / P; };
+  auto in_page = [&](int p) { return shift >= 0 ? p & (P - 1) : p % P; };
+  auto key_page = [&](int kt) -> int {
+    const int p = kt * 16 + r;
+    return (kt < tile_hi && p < kv_len && p >= lo) ? table[page_of(p)] : -1;
+  };
+  auto value_page = [&](int kt) -> int {
+    const int p = kt * 16 + 4 * g;
+    return (kt < tile_hi && p < kv_len && p + 3 >= lo) ? table[page_of(p)] : -1;
+  };
+  auto request_keys = [&](int kt, int page) {
     if constexpr (!AHEAD) return;
     const int p = kt * 16 + r;
-    int page = -1;
-    if (kt < tile_hi && p < kv_len && p >= lo) page = table[p / P];
 #pragma unroll
     for (int i = 0; i < HPW; ++i) {
       const int head = wave * HPW + i;
       const int kvh = (head < H ? head : 0) / heads_per_kv;
-      const T* k_row = keys + (((size_t)(page < 0 ? 0 : page) * a.G + kvh) * P + p % P) * D;
+      const T* k_row = keys + (((size_t)(page < 0 ? 0 : page) * a.G + kvh) * P + in_page(p)) * D;
 #pragma unroll
       for (int st = 0; st < KP; ++st) {
         const int chunk = st * 4 + g;
@@ -158,7 +169,10 @@ __global__ __launch_bounds__(WMAX * 64) void attn_mixed_kernel(MixedAttnArgs a) 
       }
     }
   };
-  if (ahead) request_keys(tile_lo);
+  int kpage = key_page(tile_lo);
+  if (ahead) request_keys(tile_lo, kpage);
+  int kpage_next = key_page(tile_lo + 1);
+  int vpage = value_page(tile_lo);
   int buf = 0;
   for (int kt = tile_lo; kt < tile_hi; ++kt, buf ^= 1) {
     const int p0 = kt * 16;
@@ -169,8 +183,7 @@ __global__ __launch_bounds__(WMAX * 64) void attn_mixed_kernel(MixedAttnArgs a) 
     f32x4 raw_own[HPW];
     {
       const int p = p0 + r;
-      int page = -1;
-      if (!ahead && p < kv_len && p >= lo) page = table[p / P];
+      const int page = kpage;
 #pragma unroll
       for (int i = 0; i < HPW; ++i) {
         const int head = wave * HPW + i;
@@ -187,7 +200,7 @@ __global__ __launch_bounds__(WMAX * 64) void attn_mixed_kernel(MixedAttnArgs a) 
             }
           } else {
             const int kvh = head / heads_per_kv;
-            const T* k_row = keys + (((size_t)(page < 0 ? 0 : page) * a.G + kvh) * P + p % P) * D;
+            const T* k_row = keys + (((size_t)(page < 0 ? 0 : page) * a.G + kvh) * P + in_page(p)) * D;
             for (int st = 0; st < steps; ++st) {
               const int chunk = st * 4 + g;
               const bool in = chunk < chunks;
@@ -203,14 +216,12 @@ __global__ __launch_bounds__(WMAX * 64) void attn_mixed_kernel(MixedAttnArgs a) 
     }
     // ---- this tile's values, then the next tile's keys: both are on their way during the mixing -----------------
     const int pv = p0 + 4 * g;
-    int vpage = -1;
-    if (pv < kv_len && pv + 3 >= lo) vpage = table[pv / P];
     Quad vq[HPW][VT];
 #pragma unroll
     for (int i = 0; i < HPW; ++i) {
       const int head = wave * HPW + i;
       const int kvh = (head < H ? head : 0) / heads_per_kv;
-      const T* v_base = values + ((size_t)(vpage < 0 ? 0 : vpage) * a.G + kvh) * E * P + pv % P;
+      const T* v_base = values + ((size_t)(vpage < 0 ? 0 : vpage) * a.G + kvh) * E * P + in_page(pv);
 #pragma unroll
       for (int dt = 0; dt < VT; ++dt) {
 #pragma unroll
@@ -218,7 +229,10 @@ __global__ __launch_bounds__(WMAX * 64) void attn_mixed_kernel(MixedAttnArgs a) 
         if (dt < dts && vpage >= 0 && head < H) vq[i][dt] = *reinterpret_cast<const Quad*>(v_base + (size_t)(dt * 16 + r) * P);
       }
     }
-    if (ahead) request_keys(kt + 1);
+    if (ahead) request_keys(kt + 1, kpage_next);
+    kpage = kpage_next;
+    kpage_next = key_page(kt + 2);
+    vpage = value_page(kt + 1);          // (this tile's quads are in registers already)
 #pragma unroll
     for (int i = 0; i < HPW; ++i) {
       const int head = wave * HPW + i;
@@ -371,6 +385,7 @@ static int mixed_dispatch(const MixedAttnArgs& args, int n_seqs, int max_q_len, 
   MixedAttnArgs a = args;
   a.q_in_lds = mx_lds_bytes<T>(a.H, a.D, true) <= 150 * 1024 ? 1 : 0;
   a.rows_kept = max_q_len == 1 ? 1 : 16;
+  a.page_shift = (a.P & (a.P - 1)) == 0 ? __builtin_ctz(a.P) : -1;
   const size_t lds = mx_lds_bytes<T>(a.H, a.D, a.q_in_lds != 0);
   TW_REQUIRE(waves <= 16 && lds <= 150 * 1024 && (hpw == 1 || a.E <= 128));
   int code;
@@ -438,7 +453,7 @@ extern "C" int tw_attn_mixed(int dtype, const void* q, long ldq, const void* key
   }
   if (n_seqs == 0) return 0;
   MixedAttnArgs a{q, ldq, keys, values, block_table, table_stride, q_start, kv_len, seq0, out, ldo, talk, sink, slopes,
-                  workspace, scale, out_scale, q_heads, kv_heads, key_dim, value_dim, page_size, window, splits, 16, 1};
+                  workspace, scale, out_scale, q_heads, kv_heads, key_dim, value_dim, page_size, window, splits, -1, 16, 1};
   if (dtype == TW_DTYPE_BF16) return mixed_dispatch<bf16_t>(a, n_seqs, max_q_len, stream);
   if (dtype == TW_DTYPE_F32) return mixed_dispatch<float>(a, n_seqs, max_q_len, stream);
   return TW_ERR_BAD_ARGUMENT;
