@@ -64,6 +64,7 @@ extern "C" int tw_add_table_rows(int dtype, float* x, const void* table, const i
 struct ConvArgs {
   const void* src; long ld_src;       // [n][ld_src], channel c at column c
   const float* norm_w;                // NORM only
+  const float* row_rinv;              // NORM: rsqrt(mean square + eps) of every row of src, or null (the block sums the rows itself)
   const float* taps;                  // [C][K]
   const float* bias;                  // [C] or null
   float* state;                       // [requests][2][K - 1][C]
@@ -74,7 +75,19 @@ struct ConvArgs {
   float eps, identity;
 };
 
-template <typename SrcT, typename OutT, bool NORM>
+__device__ __forceinline__ f32x4 conv_load4(const float* p) { return *reinterpret_cast<const f32x4*>(p); }
+__device__ __forceinline__ f32x4 conv_load4(const bf16_t* p) {
+  const bf16x4 v = *reinterpret_cast<const bf16x4*>(p);
+  return f32x4{(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
+}
+__device__ __forceinline__ void conv_store4(float* p, f32x4 v) { *reinterpret_cast<f32x4*>(p) = v; }
+__device__ __forceinline__ void conv_store4(bf16_t* p, f32x4 v) {
+  *reinterpret_cast<bf16x4*>(p) = bf16x4{(bf16_t)v[0], (bf16_t)v[1], (bf16_t)v[2], (bf16_t)v[3]};
+}
+
+// VEC: four consecutive channels a thread, 16-byte (8-byte for bfloat16) accesses; the launcher asks for it when
+// the channel count, the row strides and the pointers allow.
+template <typename SrcT, typename OutT, bool NORM, bool VEC>
 __global__ __launch_bounds__(256) void causal_conv_kernel(ConvArgs a) {
   __shared__ float red[TW_CONV_MAX_TAPS][4];
   __shared__ float rinv[TW_CONV_MAX_TAPS];
@@ -99,7 +112,13 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(ConvArgs a) {
     from_src[j] = (j < K && p >= start) ? src + (size_t)(first + p - start) * a.ld_src : nullptr;
     from_state[j] = (j < K && p < start && p >= 0) ? old_state + (size_t)(p - start + K - 1) * C : nullptr;
   }
-  if (NORM) {
+  if (NORM && a.row_rinv) {
+    if (threadIdx.x < TW_CONV_MAX_TAPS) {
+      const int j = threadIdx.x, p = pos - (K - 1) + j;
+      rinv[j] = (j < K && p >= start) ? a.row_rinv[first + p - start] : 0.f;
+    }
+    __syncthreads();
+  } else if (NORM) {
     // every block sums whole rows, whatever share of the channels it then writes
     float sums[TW_CONV_MAX_TAPS];
 #pragma unroll
@@ -127,8 +146,34 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(ConvArgs a) {
     }
     __syncthreads();
   }
-  const int share = (C + gridDim.y - 1) / gridDim.y;
+  const int share = ((C + gridDim.y - 1) / gridDim.y + 3) / 4 * 4;
   const int c_end = min(C, (int)(blockIdx.y + 1) * share);
+  if constexpr (VEC) {
+    for (int c = blockIdx.y * share + threadIdx.x * 4; c < c_end; c += blockDim.x * 4) {
+      f32x4 v[TW_CONV_MAX_TAPS];
+#pragma unroll
+      for (int j = 0; j < TW_CONV_MAX_TAPS; ++j) {
+        v[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (from_src[j]) v[j] = conv_load4(from_src[j] + c);
+        else if (from_state[j]) v[j] = conv_load4(from_state[j] + c);
+      }
+      f32x4 acc = a.bias ? conv_load4(a.bias + c) : f32x4{0.f, 0.f, 0.f, 0.f};
+      const f32x4 nw = NORM ? conv_load4(a.norm_w + c) : f32x4{1.f, 1.f, 1.f, 1.f};
+#pragma unroll
+      for (int j = 0; j < TW_CONV_MAX_TAPS; ++j) {
+        if (j < K) {
+          if (NORM && from_src[j]) v[j] = v[j] * rinv[j] * nw;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[e] += a.taps[(size_t)(c + e) * K + j] * v[j][e];
+          if (j == K - 1) acc += a.identity * v[j];
+          if (last && j >= 1) conv_store4(new_state + (size_t)(j - 1) * C + c, v[j]);
+        }
+      }
+      if (a.out) conv_store4((OutT*)a.out + (size_t)row * a.ld_out + c, acc);
+      if (a.out32) conv_store4(a.out32 + (size_t)row * a.ld_out32 + c, acc);
+    }
+    return;
+  }
   for (int c = blockIdx.y * share + threadIdx.x; c < c_end; c += blockDim.x) {
     float v[TW_CONV_MAX_TAPS];
 #pragma unroll
@@ -153,19 +198,44 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(ConvArgs a) {
   }
 }
 
+// rinv[n] = rsqrt(mean(x[n]^2) + eps): one wave a row.
+__global__ __launch_bounds__(256) void row_rinv_kernel(const float* __restrict__ x, long ld, float* __restrict__ rinv, int n, int C, float eps) {
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (row >= n) return;
+  const float* r = x + (size_t)row * ld;
+  float sum = 0.f;
+  if ((C & 3) == 0 && (ld & 3) == 0 && ((uintptr_t)x & 15) == 0) {
+    for (int c = lane * 4; c < C; c += 256) {
+      const f32x4 v = *reinterpret_cast<const f32x4*>(r + c);
+      sum += v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
+    }
+  } else {
+    for (int c = lane; c < C; c += 64) sum += r[c] * r[c];
+  }
+  sum = tw_wave_sum(sum);
+  if (lane == 0) rinv[row] = rsqrtf(sum / (float)C + eps);
+}
+
 // src_kind: 0 float32 rows, 1 rows of the compute type. norm_w non-null: RMS norm of the source rows first
 // (float32 rows only).
 extern "C" int tw_causal_conv(int dtype, int src_f32, const void* src, long ld_src, const float* norm_w, float eps,
                               const float* taps, const float* bias, float identity, float* state,
                               const int* q_start, const int* kv_len, const int* state_slots, const int* phase,
                               void* out, long ld_out, float* out32, long ld_out32, int n_tokens, int n_seqs,
-                              int C, int K, hipStream_t stream) {
+                              int C, int K, float* row_scratch, hipStream_t stream) {
   TW_REQUIRE(src && taps && state && q_start && kv_len && state_slots && phase && (out || out32));
   TW_REQUIRE(n_tokens >= 0 && n_seqs >= 1 && C > 0 && K >= 1 && K <= TW_CONV_MAX_TAPS);
   TW_REQUIRE(ld_src >= C && (!out || ld_out >= C) && (!out32 || ld_out32 >= C));
   TW_REQUIRE(!norm_w || src_f32);
   if (n_tokens == 0) return 0;
-  ConvArgs a{src, ld_src, norm_w, taps, bias, state, q_start, kv_len, state_slots, phase,
+  // many rows behind a norm: the rows' sums of squares are formed once, by a kernel of their own, instead of
+  // `taps` times over by the blocks that need them (row_scratch: n_tokens floats)
+  const float* row_rinv = nullptr;
+  if (norm_w && row_scratch && n_tokens >= 512) {
+    row_rinv_kernel<<<tw_div_up(n_tokens, 4), 256, 0, stream>>>((const float*)src, ld_src, row_scratch, n_tokens, C, eps);
+    row_rinv = row_scratch;
+  }
+  ConvArgs a{src, ld_src, norm_w, row_rinv, taps, bias, state, q_start, kv_len, state_slots, phase,
              out, ld_out, out32, ld_out32, n_seqs, C, K, eps, identity};
   const bool bf = dtype == TW_DTYPE_BF16;
   TW_REQUIRE(bf || dtype == TW_DTYPE_F32);
@@ -173,16 +243,24 @@ extern "C" int tw_causal_conv(int dtype, int src_f32, const void* src, long ld_s
   int shares = n_tokens >= 512 ? 1 : tw_div_up(C, 512);
   if (shares > 8) shares = 8;
   const dim3 n_blocks(n_tokens, shares);
+  const int esize = bf ? 2 : 4, ssize = src_f32 ? 4 : esize;
+  const bool vec = C % 4 == 0 && ld_src % 4 == 0 && (uintptr_t)src % (4 * ssize) == 0 &&
+                   (!out || (ld_out % 4 == 0 && (uintptr_t)out % (4 * esize) == 0)) &&
+                   (!out32 || (ld_out32 % 4 == 0 && (uintptr_t)out32 % 16 == 0)) && (uintptr_t)state % 16 == 0 &&
+                   (!bias || (uintptr_t)bias % 16 == 0) && (!norm_w || (uintptr_t)norm_w % 16 == 0);
+#define TW_CONV_LAUNCH(S, O, N)                                                                    \
+  do {                                                                                             \
+    if (vec) causal_conv_kernel<S, O, N, true><<<n_blocks, 256, 0, stream>>>(a);                   \
+    else causal_conv_kernel<S, O, N, false><<<n_blocks, 256, 0, stream>>>(a);                      \
+  } while (0)
   if (norm_w) {
-    if (bf) causal_conv_kernel<float, bf16_t, true><<<n_blocks, 256, 0, stream>>>(a);
-    else causal_conv_kernel<float, float, true><<<n_blocks, 256, 0, stream>>>(a);
+    if (bf) TW_CONV_LAUNCH(float, bf16_t, true); else TW_CONV_LAUNCH(float, float, true);
   } else if (src_f32) {
-    if (bf) causal_conv_kernel<float, bf16_t, false><<<n_blocks, 256, 0, stream>>>(a);
-    else causal_conv_kernel<float, float, false><<<n_blocks, 256, 0, stream>>>(a);
+    if (bf) TW_CONV_LAUNCH(float, bf16_t, false); else TW_CONV_LAUNCH(float, float, false);
   } else {
-    if (bf) causal_conv_kernel<bf16_t, bf16_t, false><<<n_blocks, 256, 0, stream>>>(a);
-    else causal_conv_kernel<float, float, false><<<n_blocks, 256, 0, stream>>>(a);
+    if (bf) TW_CONV_LAUNCH(bf16_t, bf16_t, false); else TW_CONV_LAUNCH(float, float, false);
   }
+#undef TW_CONV_LAUNCH
   return TW_LAUNCH_RESULT();
 }
 

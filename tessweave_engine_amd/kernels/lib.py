@@ -37,7 +37,7 @@ _SIGNATURES = {
     "tw_attn_prefill_workspace_floats": (L, [I, I, I, I]),
     "tw_attn_prefill": (I, [I, P, L, P, P, P, I, P, P, I, I, I, P, L, P, L, I, I, I, I, I, I, I, I, I, F, F, I, P]),
     "tw_add_table_rows": (I, [I, P, P, P, I, I, I, P, P]),
-    "tw_causal_conv": (I, [I, I, P, L, P, F, P, P, F, P, P, P, P, P, P, L, P, L, I, I, I, I, P]),
+    "tw_causal_conv": (I, [I, I, P, L, P, F, P, P, F, P, P, P, P, P, P, L, P, L, I, I, I, I, P, P]),
     "tw_gated_recurrence_workspace_floats": (L, [I, I, I]),
     "tw_gated_recurrence": (I, [I, P, L, P, L, P, L, P, P, P, P, P, L, I, I, I, I, I, F, F, P, L, P]),
     "tw_block_diagonal": (I, [I, P, L, P, P, P, L, I, I, I, I, P]),

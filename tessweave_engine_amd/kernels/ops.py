@@ -477,12 +477,14 @@ CONV_MAX_TAPS = 8
 
 
 def causal_conv(src, taps, state, q_start, kv_len, state_slots, phase, n_seqs, out=None, out32=None, norm_weight=None,
-                eps=0.0, bias=None, identity=0.0):
+                eps=0.0, bias=None, identity=0.0, row_scratch=None):
     """Causal convolution over time on each channel, with the request's last inputs as state.
 
     v_t = src_t (or its RMS norm times norm_weight, for float32 rows); out_t = identity * v_t +
     sum_j taps[:, j] * v_(t - K + 1 + j) + bias. state float32 [requests, 2, max(K - 1, 1), C]: copy
     phase[s] is read, the other copy written. out has the compute type, out32 is float32; either may be None.
+    row_scratch: float32 [>= n]; with a norm and many rows the rows' statistics are then formed once by a kernel of
+    their own.
     """
     n, C, ld_src = _rows(src, "src")
     K = taps.shape[1]
@@ -508,13 +510,17 @@ def causal_conv(src, taps, state, q_start, kv_len, state_slots, phase, n_seqs, o
         _need(bias.numel() == C and bias.dtype == torch.float32, "bias must be float32 [C]")
     _need(q_start.numel() >= n_seqs + 1 and kv_len.numel() >= n_seqs and state_slots.numel() >= n_seqs
           and phase.numel() >= n_seqs, "sequence metadata is too short")
+    use_scratch = row_scratch is not None and norm_weight is not None
+    if use_scratch:
+        _need(row_scratch.is_contiguous() and row_scratch.numel() >= n, "row_scratch must hold a float per row")
     check(library().tw_causal_conv(dtype_id(compute), 1 if src_f32 else 0, _dev(src), ld_src,
                                    _dev(norm_weight, torch.float32, "norm_weight") if norm_weight is not None else None,
                                    float(eps), _dev(taps), _dev(bias) if bias is not None else None, float(identity),
                                    _dev(state), _dev(q_start, torch.int32, "q_start"), _dev(kv_len, torch.int32, "kv_len"),
                                    _dev(state_slots, torch.int32, "state_slots"), _dev(phase, torch.int32, "phase"),
                                    _dev(out) if out is not None else None, ld_out,
-                                   _dev(out32) if out32 is not None else None, ld_out32, n, int(n_seqs), C, K, _stream()),
+                                   _dev(out32) if out32 is not None else None, ld_out32, n, int(n_seqs), C, K,
+                                   _dev(row_scratch, torch.float32, "row_scratch") if use_scratch else None, _stream()),
           "causal_conv")
 
 

@@ -112,12 +112,12 @@ def test_mixed_head_attention(device, dtype, H, G, D, E, window, T, q_len, page)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("taps,norm", [(3, True), (4, False), (1, True), (2, False)])
-def test_causal_conv_over_portions_and_reused_slots(device, dtype, taps, norm):
+@pytest.mark.parametrize("taps,norm,C", [(3, True, 40), (4, False, 40), (1, True, 38), (2, False, 38), (8, True, 38)])
+def test_causal_conv_over_portions_and_reused_slots(device, dtype, taps, norm, C):
     """Sequences in portions of 1 to 9 tokens, two at a time, in state slots that were used before."""
     from tessweave_engine_amd.kernels import ops
     g = torch.Generator().manual_seed(taps * 7 + norm)
-    C, dt = 40, tdtype(dtype)
+    dt = tdtype(dtype)
     w = torch.randn(C, taps, generator=g)
     bias = None if norm else torch.randn(C, generator=g)
     nw = 1 + 0.3 * torch.randn(C, generator=g)
@@ -373,6 +373,22 @@ def test_ways_of_cutting_agree(model):
         d.close()
     for other_run in runs[1:]:
         assert row_error(other_run, runs[0]).max() < 2e-5
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_prompt_in_one_step_then_portions(device, tmp_path, dtype):
+    """600 tokens: 520 in one step (the kernels' forms for many rows: norm statistics formed once, the recurrence
+    in chunks, attention over many tiles), then portions of 64, 15 and 1."""
+    c = CONFIGS["odd"]
+    weights = make_weights(c, seed=13)
+    folder = write_folder(tmp_path, c, weights)
+    toks = torch.randint(0, c["vocab"], (600,), generator=torch.Generator().manual_seed(4)).tolist()
+    want = plain.forward(c, weights, toks).numpy()
+    d = Driver(folder, dtype, pages=80, page_size=8)
+    got = d.run([[("a", 520)], [("a", 64)], [("a", 15)], [("a", 1)]], {"a": toks})["a"]
+    err = row_error(got, want)
+    assert err.max() < BAR[dtype], (int(err.argmax()), float(err.max()))
+    d.close()
 
 
 def test_long_decoding_past_every_window(device, tmp_path):
