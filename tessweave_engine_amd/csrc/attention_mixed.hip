@@ -63,9 +63,12 @@ static size_t mx_lds_bytes(int H, int D, bool q_in_lds) {
 }
 
 // HPW heads a wave, VT 16-column tiles of a head's values, WMAX the most waves a workgroup may have (it sets the
-// registers a lane may use), AHEAD whether key fragments are requested a tile ahead (it costs registers).
-template <typename T, int HPW, int VT, int WMAX, bool AHEAD>
+// registers a lane may use), AHEAD whether key fragments are requested a tile ahead (it costs registers), SHARE
+// whether all heads of a wave read the same key/value head (its fragments are then loaded once for all of them,
+// and everything a wave does once a key tile, page lookups, addresses, loads, is paid once for HPW heads).
+template <typename T, int HPW, int VT, int WMAX, bool AHEAD, bool SHARE>
 __global__ __launch_bounds__(WMAX * 64) void attn_mixed_kernel(MixedAttnArgs a) {
+  constexpr int KVN = SHARE ? 1 : HPW;                     // key/value heads a wave loads
   typedef typename Elem<T>::Frag Frag;
   typedef typename MxQuad<T>::Type Quad;
   constexpr int EPF = Elem<T>::kPerFrag;
@@ -141,7 +144,7 @@ __global__ __launch_bounds__(WMAX * 64) void attn_mixed_kernel(MixedAttnArgs a) 
   // (head sizes up to 128 in bfloat16, 64 in float32); longer heads load their fragments where they are used.
   constexpr int KP = AHEAD ? 4 : 1;
   const bool ahead = AHEAD && steps <= KP;
-  Frag kpre[HPW][KP];
+  Frag kpre[KVN][KP];
   // Page numbers are looked up a tile before the loads that need them, so that no load waits for a lookup.
   const int shift = a.page_shift;
   auto page_of = [&](int p) { return shift >= 0 ? p >> shift : p / P; };
@@ -158,8 +161,8 @@ __global__ __launch_bounds__(WMAX * 64) void attn_mixed_kernel(MixedAttnArgs a) 
     if constexpr (!AHEAD) return;
     const int p = kt * 16 + r;
 #pragma unroll
-    for (int i = 0; i < HPW; ++i) {
-      const int head = wave * HPW + i;
+    for (int i = 0; i < KVN; ++i) {
+      const int head = wave * HPW + i;                     // (SHARE: the wave's first head stands for all)
       const int kvh = (head < H ? head : 0) / heads_per_kv;
       const T* k_row = keys + (((size_t)(page < 0 ? 0 : page) * a.G + kvh) * P + in_page(p)) * D;
 #pragma unroll
@@ -195,7 +198,7 @@ __global__ __launch_bounds__(WMAX * 64) void attn_mixed_kernel(MixedAttnArgs a) 
             for (int st = 0; st < KP; ++st) {
               const int chunk = st * 4 + g;
               if (st < steps) {
-                tw_mma16(s, kpre[i][st], q_frag(head, chunk));
+                tw_mma16(s, kpre[SHARE ? 0 : i][st], q_frag(head, chunk));
               }
             }
           } else {
@@ -216,9 +219,9 @@ __global__ __launch_bounds__(WMAX * 64) void attn_mixed_kernel(MixedAttnArgs a) 
     }
     // ---- this tile's values, then the next tile's keys: both are on their way during the mixing -----------------
     const int pv = p0 + 4 * g;
-    Quad vq[HPW][VT];
+    Quad vq[KVN][VT];
 #pragma unroll
-    for (int i = 0; i < HPW; ++i) {
+    for (int i = 0; i < KVN; ++i) {
       const int head = wave * HPW + i;
       const int kvh = (head < H ? head : 0) / heads_per_kv;
       const T* v_base = values + ((size_t)(vpage < 0 ? 0 : vpage) * a.G + kvh) * E * P + in_page(pv);
@@ -292,7 +295,7 @@ __global__ __launch_bounds__(WMAX * 64) void attn_mixed_kernel(MixedAttnArgs a) 
 #pragma unroll
         for (int dt = 0; dt < VT; ++dt) {
           if (dt < dts) {
-            Quad v = vq[i][dt];
+            Quad v = vq[SHARE ? 0 : i][dt];
             if (!interior) {
 #pragma unroll
               for (int e = 0; e < 4; ++e)
@@ -364,9 +367,9 @@ __global__ __launch_bounds__(256) void attn_mixed_merge_kernel(MixedAttnArgs a) 
   }
 }
 
-template <typename T, int HPW, int VT, int WMAX, bool AHEAD>
+template <typename T, int HPW, int VT, int WMAX, bool AHEAD, bool SHARE>
 static int mixed_launch(const MixedAttnArgs& a, int n_seqs, int tiles, int waves, size_t lds, hipStream_t stream) {
-  auto kernel = attn_mixed_kernel<T, HPW, VT, WMAX, AHEAD>;
+  auto kernel = attn_mixed_kernel<T, HPW, VT, WMAX, AHEAD, SHARE>;
   if (lds > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
@@ -378,28 +381,32 @@ static int mixed_launch(const MixedAttnArgs& a, int n_seqs, int tiles, int waves
 template <typename T>
 static int mixed_dispatch(const MixedAttnArgs& args, int n_seqs, int max_q_len, hipStream_t stream) {
   const int tiles = tw_div_up(max_q_len, 16);
-  // One head a wave up to 16 heads; two a wave (values of up to 128 elements only: the output sums of a
-  // wave's heads live in its registers) up to 32.
-  const int hpw = args.H <= 16 ? 1 : 2;
+  // Heads a wave: one up to 8 heads, two above (workgroups of up to 8 waves up to 16 heads). What a wave does once
+  // a key tile (page lookups, addresses, loads of keys and values) is paid once for both heads where they share a
+  // key/value head, and fewer waves wait at the tile's barrier. The output sums of a wave's heads live in its registers.
+  // (measured at 2,048 tokens, heads of 128: 8 heads 164 us with one head a wave, 218 with two; 12 heads 338 and
+  // 295; 16 heads 431 and 271; four heads a wave ran out of registers and was slower than two at 16 and 32 heads)
+  const int per_kv = args.H / args.G;
+  const int hpw = args.H <= 8 ? 1 : 2;
   const int waves = tw_div_up(args.H, hpw);
+  const bool share = hpw == 2 && per_kv % 2 == 0;
   MixedAttnArgs a = args;
   a.q_in_lds = mx_lds_bytes<T>(a.H, a.D, true) <= 150 * 1024 ? 1 : 0;
   a.rows_kept = max_q_len == 1 ? 1 : 16;
   a.page_shift = (a.P & (a.P - 1)) == 0 ? __builtin_ctz(a.P) : -1;
   const size_t lds = mx_lds_bytes<T>(a.H, a.D, a.q_in_lds != 0);
-  TW_REQUIRE(waves <= 16 && lds <= 150 * 1024 && (hpw == 1 || a.E <= 128));
+  TW_REQUIRE(waves <= 16 && lds <= 150 * 1024);
   int code;
-  if (hpw == 2)
-    code = a.E <= 64 ? mixed_launch<T, 2, 4, 16, false>(a, n_seqs, tiles, waves, lds, stream)
-                     : mixed_launch<T, 2, 8, 16, false>(a, n_seqs, tiles, waves, lds, stream);
-  else if (waves <= 8)          // up to 8 heads: workgroups of up to 512 lanes, which may use twice the registers
-    code = a.E <= 64 ? mixed_launch<T, 1, 4, 8, true>(a, n_seqs, tiles, waves, lds, stream)
-         : a.E <= 128 ? mixed_launch<T, 1, 8, 8, true>(a, n_seqs, tiles, waves, lds, stream)
-                      : mixed_launch<T, 1, 16, 8, true>(a, n_seqs, tiles, waves, lds, stream);
-  else
-    code = a.E <= 64 ? mixed_launch<T, 1, 4, 16, true>(a, n_seqs, tiles, waves, lds, stream)
-         : a.E <= 128 ? mixed_launch<T, 1, 8, 16, true>(a, n_seqs, tiles, waves, lds, stream)
-                      : mixed_launch<T, 1, 16, 16, false>(a, n_seqs, tiles, waves, lds, stream);
+#define TW_MIXED(HPW_, VT_, WMAX_, AHEAD_)                                                                          \
+  (share ? mixed_launch<T, HPW_, VT_, WMAX_, AHEAD_, (HPW_ > 1)>(a, n_seqs, tiles, waves, lds, stream)               \
+         : mixed_launch<T, HPW_, VT_, WMAX_, AHEAD_, false>(a, n_seqs, tiles, waves, lds, stream))
+  if (hpw == 1)
+    code = a.E <= 64 ? TW_MIXED(1, 4, 8, true) : a.E <= 128 ? TW_MIXED(1, 8, 8, true) : TW_MIXED(1, 16, 8, true);
+  else if (waves <= 8)
+    code = a.E <= 64 ? TW_MIXED(2, 4, 8, true) : a.E <= 128 ? TW_MIXED(2, 8, 8, true) : TW_MIXED(2, 16, 8, true);
+  else                          // more than 16 heads: up to 16 waves, half the registers each
+    code = a.E <= 64 ? TW_MIXED(2, 4, 16, false) : a.E <= 128 ? TW_MIXED(2, 8, 16, false) : TW_MIXED(2, 16, 16, false);
+#undef TW_MIXED
   if (code != 0 || a.splits == 1) return code;
   attn_mixed_merge_kernel<T><<<dim3(tiles, n_seqs, a.H), 256, 0, stream>>>(a);
   return TW_LAUNCH_RESULT();
