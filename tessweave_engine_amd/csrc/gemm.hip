@@ -181,7 +181,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_lds_kernel(const T* __
       if (row >= M || col >= N / 2) continue;
       const float gv = ex[((2 * pair) * MT * 16 + row) * GROW + i];
       const float uv = ex[((2 * pair + 1) * MT * 16 + row) * GROW + i];
-      C[(size_t)row * ldc + col] = tw_from_float<OutT>(tw_silu(gv) * uv);
+      C[(size_t)row * ldc + col] = tw_from_float<OutT>(tw_glu(gv, uv, ldr));
     }
     return;
   }
@@ -434,7 +434,7 @@ __global__ __launch_bounds__(TW_CU_WAVES * 64) void gemm_stream_cu_kernel(
           if (row >= M || out0 + c >= N / 2) continue;
           const float gv = ex[(gate_wave * MT * 16 + row) * GROW + c];
           const float uv = ex[((gate_wave + 1) * MT * 16 + row) * GROW + c];
-          C[(size_t)row * ldc + out0 + c] = tw_from_float<OutT>(tw_silu(gv) * uv);
+          C[(size_t)row * ldc + out0 + c] = tw_from_float<OutT>(tw_glu(gv, uv, ldr));
         }
       }
       TW_CU_WAIT(0);
@@ -503,7 +503,7 @@ __global__ void gemm_generic_kernel(const T* __restrict__ A, long lda, const T* 
     const int gate = (col / 16) * 32 + col % 16, up = gate + 16;
     const float gv = tw_generic_dot(a, W, ldw, gate, K, shuffled) + (bias ? bias[gate] : 0.f);
     const float uv = tw_generic_dot(a, W, ldw, up, K, shuffled) + (bias ? bias[up] : 0.f);
-    C[(size_t)row * ldc + col] = tw_from_float<OutT>(tw_silu(gv) * uv);
+    C[(size_t)row * ldc + col] = tw_from_float<OutT>(tw_glu(gv, uv, ldr));
     return;
   }
   float v = tw_generic_dot(a, W, ldw, col, K, shuffled);
@@ -765,24 +765,28 @@ extern "C" int tw_linear(int dtype, int out_f32, const void* A, long lda, const 
 
 template <typename T>
 static int glu_layout(int shuffled, const T* A, long lda, const T* W, long ldw, const float* bias, T* C, long ldc,
-                      int M, int N, int K, int force, hipStream_t stream) {
+                      int M, int N, int K, int force, long code, hipStream_t stream) {
+  // (no residual in the gated form: its stride carries the activation and the factor, see tw_glu)
   if (shuffled)
-    return linear_dispatch<T, T, true, true>(A, lda, W, ldw, bias, nullptr, 0, C, ldc, nullptr, 0, M, N, K, force, stream);
-  return linear_dispatch<T, T, false, true>(A, lda, W, ldw, bias, nullptr, 0, C, ldc, nullptr, 0, M, N, K, force, stream);
+    return linear_dispatch<T, T, true, true>(A, lda, W, ldw, bias, nullptr, code, C, ldc, nullptr, 0, M, N, K, force, stream);
+  return linear_dispatch<T, T, false, true>(A, lda, W, ldw, bias, nullptr, code, C, ldc, nullptr, 0, M, N, K, force, stream);
 }
 
 // Gated linear unit: W [N, K] holds gate and up rows interleaved in blocks of 16 (N a multiple
-// of 32); C [M, N / 2] = silu(gate) * up in the input type. bias (may be null) is indexed like W's rows.
+// of 32); C [M, N / 2] = factor * act(gate) * up in the input type (act: TW_GLU_SILU or TW_GLU_GELU_TANH). bias (may be
+// null) is indexed like W's rows.
 extern "C" int tw_linear_glu(int dtype, const void* A, long lda, const void* W, long ldw, int shuffled,
-                             const float* bias, void* C, long ldc, int M, int N, int K, int force,
-                             hipStream_t stream) {
+                             const float* bias, void* C, long ldc, int M, int N, int K, int force, int act,
+                             float factor, hipStream_t stream) {
+  TW_REQUIRE(act == TW_GLU_SILU || act == TW_GLU_GELU_TANH);
+  const long code = tw_glu_code(act, factor);
   TW_REQUIRE(M >= 0 && N > 0 && N % 32 == 0 && K > 0 && lda >= K && ldc >= N / 2);
   TW_REQUIRE(weight_layout_ok(dtype, shuffled, ldw, K));
   if (M == 0) return 0;
   if (dtype == TW_DTYPE_F32)
-    return glu_layout<float>(shuffled, (const float*)A, lda, (const float*)W, ldw, bias, (float*)C, ldc, M, N, K, force, stream);
+    return glu_layout<float>(shuffled, (const float*)A, lda, (const float*)W, ldw, bias, (float*)C, ldc, M, N, K, force, code, stream);
   if (dtype == TW_DTYPE_BF16)
-    return glu_layout<bf16_t>(shuffled, (const bf16_t*)A, lda, (const bf16_t*)W, ldw, bias, (bf16_t*)C, ldc, M, N, K, force, stream);
+    return glu_layout<bf16_t>(shuffled, (const bf16_t*)A, lda, (const bf16_t*)W, ldw, bias, (bf16_t*)C, ldc, M, N, K, force, code, stream);
   return TW_ERR_BAD_ARGUMENT;
 }
 

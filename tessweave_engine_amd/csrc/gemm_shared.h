@@ -6,6 +6,27 @@
 
 __device__ __forceinline__ float tw_silu(float g) { return g / (1.0f + expf(-g)); }
 
+// The gated form act(gate) * up adds no residual, so the residual's row stride is free there and carries which
+// activation the gate passes and a factor for the product: 0 is SiLU and 1 (what every caller before the second
+// activation passed); otherwise bits 32.. name the activation (1: the tanh form of gelu) and the low 32 bits are
+// the factor as a float. The factor is applied in float32 before the one rounding to the output type.
+#define TW_GLU_SILU 0
+#define TW_GLU_GELU_TANH 1
+static inline long tw_glu_code(int act, float factor) {
+  if (act == TW_GLU_SILU && factor == 1.0f) return 0;
+  unsigned bits;
+  __builtin_memcpy(&bits, &factor, 4);
+  return ((long)(act + 1) << 32) | (long)bits;
+}
+__device__ __forceinline__ float tw_glu(float g, float u, long code) {
+  if (code == 0) return tw_silu(g) * u;
+  const float factor = __uint_as_float((unsigned)(code & 0xffffffffL));
+  const int act = (int)(code >> 32) - 1;
+  const float a = act == TW_GLU_GELU_TANH ? 0.5f * g * (1.f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)))
+                                          : tw_silu(g);
+  return factor * a * u;
+}
+
 // Sum of split-K partial sums partial[split][M][N], in split order, then bias and residual.
 template <typename OutT>
 __global__ void splitk_reduce_kernel(const float* __restrict__ partial, int splits,

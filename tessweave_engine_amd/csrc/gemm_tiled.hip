@@ -87,7 +87,7 @@ __device__ __forceinline__ void tw_tiled_epilogue(f32x16 (&acc)[WM][WN], char* l
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           if (bias) { gv[e] += bias[col + e]; uv[e] += bias[col + 16 + e]; }
-          v[e] = tw_silu(gv[e]) * uv[e];
+          v[e] = tw_glu(gv[e], uv[e], ldr);
         }
         OutT* dst = C + (size_t)row * ldc + (n0 + wn0) / 2 + (og >> 1) * 16 + (og & 1) * 8;
         if (ldc % 8 == 0 && (uintptr_t)C % 16 == 0) {

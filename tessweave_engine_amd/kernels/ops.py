@@ -282,9 +282,14 @@ def interleave_glu_rows(gate, up):
     return torch.stack([gate.reshape(n // 16, 16, *rest), up.reshape(n // 16, 16, *rest)], 1).reshape(2 * n, *rest).contiguous()
 
 
-def linear_glu(x, weight, out, bias=None, force=0):
-    """out[m, n/2] = silu(x @ gate.T) * (x @ up.T), weight [n, k] holding gate and up rows
-    interleaved by `interleave_glu_rows` (row-major or shuffled); out has x's type."""
+GLU_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+
+
+def linear_glu(x, weight, out, bias=None, force=0, activation="silu", factor=1.0):
+    """out[m, n/2] = factor * act(x @ gate.T) * (x @ up.T), weight [n, k] holding gate and up rows
+    interleaved by `interleave_glu_rows` (row-major or shuffled); out has x's type. act is SiLU or the tanh
+    form of gelu; the factor is applied in float32 before the rounding."""
+    _need(activation in GLU_ACTIVATIONS, f"activation must be one of {sorted(GLU_ACTIVATIONS)}")
     m, k, lda = _rows(x, "x")
     n, k2, w_ptr, ldw, shuffled, w_dtype = _weight_args(weight)
     mo, no, ldc = _rows(out, "out")
@@ -295,7 +300,8 @@ def linear_glu(x, weight, out, bias=None, force=0):
         _need(bias.numel() == n, "bias has the wrong size")
     check(library().tw_linear_glu(dtype_id(x.dtype), _dev(x), lda, w_ptr, ldw, shuffled,
                                   _dev(bias, torch.float32, "bias") if bias is not None else None,
-                                  _dev(out), ldc, m, n, k, force, _stream()), "linear_glu")
+                                  _dev(out), ldc, m, n, k, force, GLU_ACTIVATIONS[activation], float(factor), _stream()),
+          "linear_glu")
     return out
 
 

@@ -44,9 +44,10 @@ class GatedFeedForward(FeedForward):
     """x += out_scale * down( act(gate(h)) * up(h) ) with a choice of activation and of tensor names.
 
     activation "silu" is `SwiGLU`'s arithmetic; "gelu_tanh" is 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))).
-    The gelu form multiplies in a kernel of its own after one packed gate|up product (the fused epilogue of the
-    matrix kernels is SiLU's); out_scale is folded into that multiplication, before the rounding to the compute
-    type, so the down projection adds straight into the residual stream.
+    Gate and up rows are interleaved so that the matrix kernels' gated epilogue forms act(gate) * up (where the
+    intermediate size is no multiple of 16 a kernel of its own multiplies after one packed product); out_scale is
+    folded into that multiplication, before the rounding to the compute type, so the down projection adds straight
+    into the residual stream.
     """
 
     def __init__(self, names, hidden, intermediate, activation="gelu_tanh", out_scale=1.0, suffix=".weight"):
@@ -54,7 +55,8 @@ class GatedFeedForward(FeedForward):
             raise ValueError("GatedFeedForward computes gelu_tanh; SwiGLU is the SiLU part")
         gate, up, down = names
         self.hidden, self.intermediate, self.out_scale = int(hidden), int(intermediate), float(out_scale)
-        self.gate_up = Linear([gate, up], hidden, [intermediate, intermediate], suffixes=(suffix, ".bias"))
+        self.activation = activation
+        self.gate_up = Linear([gate, up], hidden, [intermediate, intermediate], glu=True, suffixes=(suffix, ".bias"))
         self.down = Linear([down], intermediate, [hidden], suffixes=(suffix, ".bias"))
 
     def parts(self):
@@ -69,9 +71,12 @@ class GatedFeedForward(FeedForward):
 
     def forward(self, ctx, h, x):
         n = h.shape[0]
-        gu = ctx.scratch("ffn.gate_up", (n, 2 * self.intermediate))
-        self.gate_up.forward(ctx, h, gu)
         act = ctx.scratch("ffn.act", (n, self.intermediate))
-        ops.gelu_mul(gu, act, self.out_scale)
+        if self.gate_up.gated:
+            self.gate_up.forward_glu(ctx, h, act, activation=self.activation, factor=self.out_scale)
+        else:
+            gu = ctx.scratch("ffn.gate_up", (n, 2 * self.intermediate))
+            self.gate_up.forward(ctx, h, gu)
+            ops.gelu_mul(gu, act, self.out_scale)
         self.down.forward(ctx, act, x, residual=x)
         return None

@@ -152,9 +152,10 @@ class Linear(Part):
         w = self.weights[i]
         return w.to_rows() if isinstance(w, ops.ShuffledWeight) else w
 
-    def forward_glu(self, ctx, x, out):
-        """out [n, rows of one matrix] = silu(x @ gate.T + b) * (x @ up.T + b), in x's type (needs `gated`)."""
-        return ops.linear_glu(x, self.weights[0], out, bias=self.biases[0] if self.biases else None)
+    def forward_glu(self, ctx, x, out, activation="silu", factor=1.0):
+        """out [n, rows of one matrix] = factor * act(x @ gate.T + b) * (x @ up.T + b), in x's type (needs `gated`)."""
+        return ops.linear_glu(x, self.weights[0], out, bias=self.biases[0] if self.biases else None,
+                              activation=activation, factor=factor)
 
     def forward(self, ctx, x, out, residual=None):
         """out[:, columns] = x @ W.T (+ bias) (+ residual); out may be float32 or x's type."""

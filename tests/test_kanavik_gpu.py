@@ -220,6 +220,25 @@ def test_block_diagonal_product(device, dtype, n, blocks, n_in, n_out):
     assert torch.allclose(out.cpu().double(), want, atol=tol, rtol=tol)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("rows", [3, 40, 300])
+def test_gated_product_with_gelu_and_a_factor(device, dtype, rows):
+    """The matrix kernels' gated epilogue with the tanh form of gelu (few rows, 17-64 rows, tiled) and shuffled weights."""
+    from tessweave_engine_amd.kernels import ops
+    g = torch.Generator().manual_seed(rows)
+    dt = tdtype(dtype)
+    k, inter = 96, 160
+    x = torch.randn(rows, k, generator=g).to(dt)
+    gate = (torch.randn(inter, k, generator=g) / math.sqrt(k)).to(dt)
+    up = (torch.randn(inter, k, generator=g) / math.sqrt(k)).to(dt)
+    want = 0.7 * plain.gelu_tanh(x.double() @ gate.double().T) * (x.double() @ up.double().T)
+    packed = ops.shuffle_weight(ops.interleave_glu_rows(gate.to(device), up.to(device)))
+    out = torch.empty(rows, inter, dtype=dt, device=device)
+    ops.linear_glu(x.to(device), packed, out, activation="gelu_tanh", factor=0.7)
+    tol = 2e-5 if dtype == "float32" else 2e-2
+    assert torch.allclose(out.cpu().double(), want, atol=tol, rtol=tol)
+
+
 def test_small_kernels(device):
     from tessweave_engine_amd.kernels import ops
     g = torch.Generator().manual_seed(9)
