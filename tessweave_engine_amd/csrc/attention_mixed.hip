@@ -66,14 +66,17 @@ static size_t mx_lds_bytes(int H, int D, bool q_in_lds) {
 // registers a lane may use), AHEAD whether key fragments are requested a tile ahead (it costs registers), SHARE
 // whether all heads of a wave read the same key/value head (its fragments are then loaded once for all of them,
 // and everything a wave does once a key tile, page lookups, addresses, loads, is paid once for HPW heads).
-template <typename T, int HPW, int VT, int WMAX, bool AHEAD, bool SHARE>
+// EXACT: the key size is exactly what four MFMA steps of fragments hold (128 in bfloat16, 64 in float32) and the
+// value size is 16 VT: sizes and loop bounds are then compile-time constants.
+template <typename T, int HPW, int VT, int WMAX, bool AHEAD, bool SHARE, bool EXACT>
 __global__ __launch_bounds__(WMAX * 64) void attn_mixed_kernel(MixedAttnArgs a) {
   constexpr int KVN = SHARE ? 1 : HPW;                     // key/value heads a wave loads
   typedef typename Elem<T>::Frag Frag;
   typedef typename MxQuad<T>::Type Quad;
   constexpr int EPF = Elem<T>::kPerFrag;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-  const int H = a.H, D = a.D, E = a.E, P = a.P;
+  const int H = a.H, P = a.P;
+  const int D = EXACT ? 16 * Elem<T>::kPerFrag : a.D, E = EXACT ? 16 * VT : a.E;
   const size_t qrow = mx_q_row<T>(D);
   T* lds_q = (T*)lds_raw;
   size_t q_bytes = a.q_in_lds ? (size_t)H * 16 * qrow * sizeof(T) : 0;
@@ -93,7 +96,7 @@ __global__ __launch_bounds__(WMAX * 64) void attn_mixed_kernel(MixedAttnArgs a) 
   const int t_row = r < n_rows ? pos0 + r : -1;
   const int* table = a.block_table + (size_t)seq * a.table_stride;
   const int heads_per_kv = H / a.G;
-  const int chunks = D / EPF, steps = (chunks + 3) / 4, dts = E / 16;
+  const int chunks = EXACT ? 16 : D / EPF, steps = EXACT ? 4 : (chunks + 3) / 4, dts = EXACT ? VT : E / 16;
 
   // ---- stage the tile's queries and the mixing matrix ------------------------------------------------
   for (int i = threadIdx.x; i < (a.q_in_lds ? H * 16 * chunks : 0); i += blockDim.x) {
@@ -138,6 +141,9 @@ __global__ __launch_bounds__(WMAX * 64) void attn_mixed_kernel(MixedAttnArgs a) 
     if (a.q_in_lds) return *reinterpret_cast<const Frag*>(lds_q + ((size_t)head * 16 + r) * qrow + chunk * EPF);
     return r < n_rows ? tw_load_frag(q_global + (size_t)head * D + chunk * EPF) : Elem<T>::zero();
   };
+  // Loads carry no condition on the page: a key outside the sequence or the window is read from page 0 (every
+  // pool has one), its score is selected away and its value set to zero by the masks of the edge tile it lies
+  // in (a tile that is not an edge tile has no such key), so whatever that page holds never reaches a result.
   // The K fragments of a key tile are requested one tile ahead (while the tile before is mixed and multiplied
   // with its values), the V quads of a tile before the barrier that publishes its raw scores: a tile then waits
   // for memory once, not twice, and mostly not at all. KP fragments a head fit the registers kept for that
@@ -168,7 +174,7 @@ __global__ __launch_bounds__(WMAX * 64) void attn_mixed_kernel(MixedAttnArgs a) 
 #pragma unroll
       for (int st = 0; st < KP; ++st) {
         const int chunk = st * 4 + g;
-        kpre[i][st] = (page >= 0 && head < H && chunk < chunks) ? tw_load_frag(k_row + chunk * EPF) : Elem<T>::zero();
+        kpre[i][st] = chunk < chunks ? tw_load_frag(k_row + chunk * EPF) : Elem<T>::zero();
       }
     }
   };
@@ -227,9 +233,7 @@ __global__ __launch_bounds__(WMAX * 64) void attn_mixed_kernel(MixedAttnArgs a) 
       const T* v_base = values + ((size_t)(vpage < 0 ? 0 : vpage) * a.G + kvh) * E * P + in_page(pv);
 #pragma unroll
       for (int dt = 0; dt < VT; ++dt) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) vq[i][dt][e] = tw_from_float<T>(0.f);
-        if (dt < dts && vpage >= 0 && head < H) vq[i][dt] = *reinterpret_cast<const Quad*>(v_base + (size_t)(dt * 16 + r) * P);
+        if (dt < dts) vq[i][dt] = *reinterpret_cast<const Quad*>(v_base + (size_t)(dt * 16 + r) * P);
       }
     }
     if (ahead) request_keys(kt + 1, kpage_next);
@@ -367,9 +371,9 @@ __global__ __launch_bounds__(256) void attn_mixed_merge_kernel(MixedAttnArgs a) 
   }
 }
 
-template <typename T, int HPW, int VT, int WMAX, bool AHEAD, bool SHARE>
+template <typename T, int HPW, int VT, int WMAX, bool AHEAD, bool SHARE, bool EXACT = false>
 static int mixed_launch(const MixedAttnArgs& a, int n_seqs, int tiles, int waves, size_t lds, hipStream_t stream) {
-  auto kernel = attn_mixed_kernel<T, HPW, VT, WMAX, AHEAD, SHARE>;
+  auto kernel = attn_mixed_kernel<T, HPW, VT, WMAX, AHEAD, SHARE, EXACT>;
   if (lds > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
@@ -397,9 +401,14 @@ static int mixed_dispatch(const MixedAttnArgs& args, int n_seqs, int max_q_len, 
   const size_t lds = mx_lds_bytes<T>(a.H, a.D, a.q_in_lds != 0);
   TW_REQUIRE(waves <= 16 && lds <= 150 * 1024);
   int code;
+  // (the sizes of most models: compile-time instances for values of 128 beside keys of four MFMA steps)
+  const bool exact = a.D == 16 * Elem<T>::kPerFrag && a.E == 128;
 #define TW_MIXED(HPW_, VT_, WMAX_, AHEAD_)                                                                          \
-  (share ? mixed_launch<T, HPW_, VT_, WMAX_, AHEAD_, (HPW_ > 1)>(a, n_seqs, tiles, waves, lds, stream)               \
-         : mixed_launch<T, HPW_, VT_, WMAX_, AHEAD_, false>(a, n_seqs, tiles, waves, lds, stream))
+  (exact && VT_ == 8 && AHEAD_                                                                                      \
+     ? (share ? mixed_launch<T, HPW_, VT_, WMAX_, AHEAD_, (HPW_ > 1), (VT_ == 8 && AHEAD_)>(a, n_seqs, tiles, waves, lds, stream)  \
+              : mixed_launch<T, HPW_, VT_, WMAX_, AHEAD_, false, (VT_ == 8 && AHEAD_)>(a, n_seqs, tiles, waves, lds, stream))      \
+     : (share ? mixed_launch<T, HPW_, VT_, WMAX_, AHEAD_, (HPW_ > 1)>(a, n_seqs, tiles, waves, lds, stream)          \
+              : mixed_launch<T, HPW_, VT_, WMAX_, AHEAD_, false>(a, n_seqs, tiles, waves, lds, stream)))
   if (hpw == 1)
     code = a.E <= 64 ? TW_MIXED(1, 4, 8, true) : a.E <= 128 ? TW_MIXED(1, 8, 8, true) : TW_MIXED(1, 16, 8, true);
   else if (waves <= 8)
@@ -428,7 +437,7 @@ extern "C" int tw_attn_mixed_splits(int n_seqs, int max_kv_len) {
 extern "C" int tw_attn_mixed_prefill_splits(int n_tokens, int n_seqs, int max_kv_len) {
   const int tiles = tw_div_up(n_tokens, 16) + n_seqs;
   const int key_tiles = tw_div_up(max_kv_len, 16);
-  int s = 320 / (tiles > 0 ? tiles : 1);
+  int s = 384 / (tiles > 0 ? tiles : 1);
   if (s > key_tiles / 8) s = key_tiles / 8;
   if (s > 8) s = 8;
   return s < 1 ? 1 : s;

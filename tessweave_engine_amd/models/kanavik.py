@@ -152,7 +152,9 @@ def build_kanavik(config: KanavikConfig, packed=True):
             ffn_in = CausalConv(p + "canon2", C, c.canon_taps, "canon2", identity=1.0,
                                 norm=RMSNorm(p + "norm2", C, c.norm_eps, suffix=""))
         side = TokenSideInput(p + "side.", table, i, C, c.side_dim, c.norm_eps, owns_table=i == 0) if table else None
-        blocks.append(DepthMixedBlock(i, L, C, mixer_in, mixer, ffn_in, ffn, side, side_mult=m, mix_name=p + "dwa"))
+        unused = () if ffn is not None else (p + "norm2", p + "canon2")
+        blocks.append(DepthMixedBlock(i, L, C, mixer_in, mixer, ffn_in, ffn, side, side_mult=m, mix_name=p + "dwa",
+                                      unused_names=unused))
     final_norm = RMSNorm("final.norm", C, c.norm_eps, suffix="")
     head = OutputHead("head", c.vocab_size, C, suffix="")
     return DecoderModel(c, embedding, blocks, final_norm, head)

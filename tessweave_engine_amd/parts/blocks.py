@@ -60,7 +60,10 @@ class DepthMixedBlock(Block):
     HISTORY_TAG = "depth.history"
 
     def __init__(self, layer, n_layers, hidden, mixer_in, mixer, ffn_in=None, ffn=None, side=None, side_mult=1.0,
-                 mix_name=None):
+                 mix_name=None, unused_names=()):
+        """unused_names: tensors a checkpoint may hold for this layer that nothing reads (the norm and convolution
+        of a feed-forward the layer does not have): accepted if present, never required."""
+        self.unused_names = tuple(unused_names)
         self.layer, self.n_layers, self.hidden = int(layer), int(n_layers), int(hidden)
         self.mixer_in, self.mixer, self.ffn_in, self.ffn, self.side = mixer_in, mixer, ffn_in, ffn, side
         self.side_mult, self.mix_name = float(side_mult), mix_name
@@ -73,6 +76,7 @@ class DepthMixedBlock(Block):
         specs = [s for p in self.parts() for s in p.tensor_specs()]
         if self.mix_name:
             specs.append(TensorSpec(self.mix_name, (self.layer + 2,), VECTOR, AVERAGE))
+        specs += [TensorSpec(name, (1,), VECTOR, optional_alias_of="(unused)") for name in self.unused_names]
         return specs
 
     def bind(self, tensors, dtype, device):

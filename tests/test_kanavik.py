@@ -18,8 +18,11 @@ def test_config_registry_and_tensor_names(name, tmp_path):
     assert config.architecture == "Kanavik" and config.vocab_size == c["vocab"]
     assert config_from_dict(config.to_dict()) == config
     model = build_model(config)
-    specs = {s.name: s.shape for s in model.tensor_specs()}
+    specs = {s.name: s.shape for s in model.tensor_specs() if s.optional_alias_of is None}
     assert specs == tensor_shapes(c)
+    # a layer without a feed-forward may still bring its second norm and convolution: accepted, never required
+    spare = sorted(s.name for s in model.tensor_specs() if s.optional_alias_of is not None)
+    assert spare == sorted(f"l{i}.{t}" for i, lay in enumerate(c["layers"]) if not lay["mlp"] for t in ("norm2", "canon2"))
     folder = write_folder(tmp_path, c, make_weights(c, 0))
     assert read_model_config(folder) == config
 
