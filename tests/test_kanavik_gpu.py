@@ -183,10 +183,10 @@ def test_gated_recurrence_carries_its_state(device, dtype):
     state = torch.zeros(2, R, device=device)
     state[0] = float("nan")                                # another request's slot
     got, at = [], 0
-    for n in (1, 5, 2, 1, 17, 14, 64, 65, 200, 31):          # portions of one chunk, of exactly one, and of several
+    for n in (1, 5, 2, 1, 17, 14, 32, 33, 64, 200, 31):      # portions of one chunk, of exactly one, and of several
         out = torch.full((n, R + 3), float("nan"), dtype=dt, device=device)
         floats = ops.gated_recurrence_workspace_floats(1, n, R)
-        assert (floats > 0) == (n > 64)
+        assert (floats > 0) == (n > 32)
         ws = torch.full((max(floats, 1),), float("nan"), device=device)
         ops.gated_recurrence(gates[at:at + n].contiguous().to(device), u[at:at + n].contiguous().to(device),
                              branch[at:at + n].to(dt).to(device), lam.to(device), state,
