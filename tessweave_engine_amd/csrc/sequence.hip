@@ -198,6 +198,89 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(ConvArgs a) {
   }
 }
 
+// The same convolution for steps of many rows: a block takes TW_CONV_TILE consecutive rows of the flat batch and
+// walks them in order, four channels a thread, keeping the last K - 1 inputs in registers: a row is read once
+// (plus K - 1 rows where a tile or a sequence's portion begins) instead of K times. With a norm the rows'
+// statistics come from `row_rinv`. What a row reads and writes is exactly what `causal_conv_kernel` reads and
+// writes for it.
+#define TW_CONV_TILE 8
+template <typename SrcT, typename OutT, bool NORM>
+__global__ __launch_bounds__(256) void causal_conv_tile_kernel(ConvArgs a, int n_tokens) {
+  __shared__ int info[TW_CONV_TILE][5];                   // per row of the tile: first row, start, length, slot, phase
+  const int row0 = blockIdx.x * TW_CONV_TILE;
+  const int rows = min(TW_CONV_TILE, n_tokens - row0);
+  if (threadIdx.x < rows) {
+    const int s = tw_seq_of_row(a.q_start, a.n_seqs, row0 + threadIdx.x);
+    const int first = a.q_start[s], len = a.kv_len[s];
+    info[threadIdx.x][0] = first;
+    info[threadIdx.x][1] = len - (a.q_start[s + 1] - first);
+    info[threadIdx.x][2] = len;
+    info[threadIdx.x][3] = a.state_slots[s];
+    info[threadIdx.x][4] = a.phase[s] & 1;
+  }
+  __syncthreads();
+  const int K = a.K, C = a.C;
+  const SrcT* src = (const SrcT*)a.src;
+  for (int c = threadIdx.x * 4; c < C; c += blockDim.x * 4) {
+    f32x4 w[TW_CONV_MAX_TAPS];                            // w[j][e]: tap j of channel c + e
+#pragma unroll
+    for (int j = 0; j < TW_CONV_MAX_TAPS; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) w[j][e] = j < K ? a.taps[(size_t)(c + e) * K + j] : 0.f;
+    const f32x4 bias = a.bias ? conv_load4(a.bias + c) : f32x4{0.f, 0.f, 0.f, 0.f};
+    const f32x4 nw = NORM ? conv_load4(a.norm_w + c) : f32x4{1.f, 1.f, 1.f, 1.f};
+    f32x4 v[TW_CONV_MAX_TAPS];                            // v[j]: the input that meets tap j; v[K - 1] the current row's
+    for (int i = 0; i < rows; ++i) {
+      const int row = row0 + i;
+      const int first = info[i][0], start = info[i][1], len = info[i][2];
+      const int pos = start + (row - first);
+      const float* old_state = a.state + ((size_t)info[i][3] * 2 + info[i][4]) * (size_t)(K - 1) * C;
+      if (i == 0 || row == first) {
+        // a tile or a portion begins: the earlier inputs come from this step's rows, the state, or nothing
+#pragma unroll
+        for (int j = 0; j < TW_CONV_MAX_TAPS - 1; ++j) {
+          v[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+          const int p = pos - (K - 1) + j;
+          if (j < K - 1) {
+            if (p >= start) {
+              const int r = first + p - start;
+              v[j] = conv_load4(src + (size_t)r * a.ld_src + c);
+              if (NORM) v[j] = v[j] * a.row_rinv[r] * nw;
+            } else if (p >= 0) {
+              v[j] = conv_load4(old_state + (size_t)(p - start + K - 1) * C + c);
+            }
+          }
+        }
+      }
+      f32x4 cur = conv_load4(src + (size_t)row * a.ld_src + c);
+      if (NORM) cur = cur * a.row_rinv[row] * nw;
+      f32x4 acc = bias + a.identity * cur;
+#pragma unroll
+      for (int j = 0; j < TW_CONV_MAX_TAPS - 1; ++j)
+        if (j < K - 1) acc += w[j] * v[j];
+      // (the current row meets the last tap, whose index is only known at run time)
+#pragma unroll
+      for (int j = 0; j < TW_CONV_MAX_TAPS; ++j)
+        if (j == K - 1) acc += w[j] * cur;
+      if (a.out) conv_store4((OutT*)a.out + (size_t)row * a.ld_out + c, acc);
+      if (a.out32) conv_store4(a.out32 + (size_t)row * a.ld_out32 + c, acc);
+      // shift: what met tap j + 1 meets tap j for the next row
+#pragma unroll
+      for (int j = 0; j < TW_CONV_MAX_TAPS - 2; ++j)
+        if (j < K - 2) v[j] = v[j + 1];
+#pragma unroll
+      for (int j = 0; j < TW_CONV_MAX_TAPS - 1; ++j)
+        if (j == K - 2) v[j] = cur;
+      if (pos == len - 1) {
+        float* new_state = a.state + ((size_t)info[i][3] * 2 + (1 - info[i][4])) * (size_t)(K - 1) * C;
+#pragma unroll
+        for (int j = 0; j < TW_CONV_MAX_TAPS - 1; ++j)
+          if (j < K - 1) conv_store4(new_state + (size_t)j * C + c, v[j]);
+      }
+    }
+  }
+}
+
 // rinv[n] = rsqrt(mean(x[n]^2) + eps): one wave a row.
 __global__ __launch_bounds__(256) void row_rinv_kernel(const float* __restrict__ x, long ld, float* __restrict__ rinv, int n, int C, float eps) {
   const int row = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
@@ -248,9 +331,11 @@ extern "C" int tw_causal_conv(int dtype, int src_f32, const void* src, long ld_s
                    (!out || (ld_out % 4 == 0 && (uintptr_t)out % (4 * esize) == 0)) &&
                    (!out32 || (ld_out32 % 4 == 0 && (uintptr_t)out32 % 16 == 0)) && (uintptr_t)state % 16 == 0 &&
                    (!bias || (uintptr_t)bias % 16 == 0) && (!norm_w || (uintptr_t)norm_w % 16 == 0);
+  const bool tiled = vec && n_tokens >= 512 && (!norm_w || row_rinv);
 #define TW_CONV_LAUNCH(S, O, N)                                                                    \
   do {                                                                                             \
-    if (vec) causal_conv_kernel<S, O, N, true><<<n_blocks, 256, 0, stream>>>(a);                   \
+    if (tiled) causal_conv_tile_kernel<S, O, N><<<tw_div_up(n_tokens, TW_CONV_TILE), 256, 0, stream>>>(a, n_tokens); \
+    else if (vec) causal_conv_kernel<S, O, N, true><<<n_blocks, 256, 0, stream>>>(a);              \
     else causal_conv_kernel<S, O, N, false><<<n_blocks, 256, 0, stream>>>(a);                      \
   } while (0)
   if (norm_w) {

@@ -167,6 +167,60 @@ def test_causal_conv_over_portions_and_reused_slots(device, dtype, taps, norm, C
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("taps,norm", [(4, True), (3, False), (1, True), (8, False), (2, True)])
+def test_causal_conv_of_many_rows(device, dtype, taps, norm):
+    """A step of 640 rows (the kernel that walks tiles of rows): a sequence that starts in it, one that goes on from
+    its state (whose first tokens come mid-tile), one of two tokens, one of one token that began steps ago."""
+    from tessweave_engine_amd.kernels import ops
+    g = torch.Generator().manual_seed(taps + 10 * norm)
+    C, dt = 48, tdtype(dtype)
+    w = torch.randn(C, taps, generator=g)
+    bias = None if norm else torch.randn(C, generator=g)
+    nw = 1 + 0.3 * torch.randn(C, generator=g)
+    lengths, before = [300, 331, 2, 7], [0, 5, 0, 6]              # tokens in all, of which in an earlier step
+    seqs = [torch.randn(n, C, generator=g) for n in lengths]
+    if not norm:
+        seqs = [s.to(dt).float() for s in seqs]
+    want = []
+    for s in seqs:
+        v = plain.rms_norm(s.double(), nw.double(), 1e-5) if norm else s.double()
+        want.append((v if norm else 0) + plain.causal_conv(v, w.double()) + (0 if norm else bias.double()))
+    state = torch.zeros(4, 2, max(taps - 1, 1), C, device=device)
+    slots = torch.tensor([3, 1, 0, 2], dtype=torch.int32, device=device)
+
+    def step(parts, phases):
+        rows = torch.cat([seqs[s][lo:hi] for s, lo, hi in parts])
+        src = rows.to(device) if norm else rows.to(dt).to(device)
+        q_start = torch.tensor(np.cumsum([0] + [hi - lo for _, lo, hi in parts]), dtype=torch.int32, device=device)
+        kv_len = torch.tensor([hi for _, _, hi in parts], dtype=torch.int32, device=device)
+        out32 = torch.empty(len(rows), C, device=device)
+        out = torch.empty(len(rows), C, dtype=dt, device=device)
+        scratch = torch.empty(len(rows), device=device)
+        ops.causal_conv(src, w.to(device), state, q_start, kv_len, slots[[s for s, _, _ in parts]].contiguous(),
+                        torch.tensor(phases, dtype=torch.int32, device=device), len(parts), out=out, out32=out32,
+                        norm_weight=nw.to(device) if norm else None, eps=1e-5, bias=bias.to(device) if bias is not None else None,
+                        identity=1.0 if norm else 0.0, row_scratch=scratch)
+        assert torch.allclose(out.float().cpu(), out32.to(dt).float().cpu())
+        return out32.cpu()
+
+    step([(1, 0, 5), (3, 0, 6)], [0, 0])                              # the earlier step of sequences 1 and 3
+    got = step([(0, 0, 300), (1, 5, 331), (2, 0, 2), (3, 6, 7)], [0, 1, 0, 1])
+    at = 0
+    for s, lo, hi in [(0, 0, 300), (1, 5, 331), (2, 0, 2), (3, 6, 7)]:
+        assert torch.allclose(got[at:at + hi - lo].double(), want[s][lo:hi], atol=2e-5, rtol=2e-5), s
+        at += hi - lo
+    # and the state it left: one more token of sequence 1 from a short step
+    extra = torch.randn(1, C, generator=g)
+    if not norm:
+        extra = extra.to(dt).float()
+    seqs[1] = torch.cat([seqs[1], extra])
+    v = plain.rms_norm(seqs[1].double(), nw.double(), 1e-5) if norm else seqs[1].double()
+    full = (v if norm else 0) + plain.causal_conv(v, w.double()) + (0 if norm else bias.double())
+    got = step([(1, 331, 332)], [0])
+    assert torch.allclose(got.double(), full[331:332], atol=2e-5, rtol=2e-5)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_gated_recurrence_carries_its_state(device, dtype):
     from tessweave_engine_amd.kernels import ops
     g = torch.Generator().manual_seed(5)
