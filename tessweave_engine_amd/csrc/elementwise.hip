@@ -285,23 +285,25 @@ extern "C" int tw_rmsnorm(int out_dtype, float* x, const float* w, void* out, co
   return TW_LAUNCH_RESULT();
 }
 
-// ---- rotary tables: cos/sin[n, j] of angle = float(position[n]) * inv_freq[j] -----
+// ---- rotary tables: cos/sin[n, j] of angle = float(position[n]) * inv_freq[j], times `magnitude` -----
+// (1 for the plain encoding; encodings that stretch their frequencies for longer contexts also scale both tables)
 __global__ void rope_table_kernel(const int* __restrict__ positions, const float* __restrict__ inv_freq,
-                                  float* __restrict__ cos_out, float* __restrict__ sin_out, int n, int half) {
+                                  float* __restrict__ cos_out, float* __restrict__ sin_out, int n, int half,
+                                  float magnitude) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n * half) return;
   const int t = i / half, j = i % half;
   const float angle = (float)positions[t] * inv_freq[j];
-  cos_out[i] = cosf(angle);
-  sin_out[i] = sinf(angle);
+  cos_out[i] = cosf(angle) * magnitude;
+  sin_out[i] = sinf(angle) * magnitude;
 }
 
 extern "C" int tw_rope_table(const int* positions, const float* inv_freq, float* cos_out, float* sin_out,
-                             int n, int half, hipStream_t stream) {
+                             int n, int half, float magnitude, hipStream_t stream) {
   TW_REQUIRE(n >= 0 && half > 0);
   if (n == 0) return 0;
   rope_table_kernel<<<tw_div_up((long)n * half, 256), 256, 0, stream>>>(positions, inv_freq, cos_out,
-                                                                       sin_out, n, half);
+                                                                       sin_out, n, half, magnitude);
   return TW_LAUNCH_RESULT();
 }
 

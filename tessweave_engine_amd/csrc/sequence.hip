@@ -688,3 +688,72 @@ extern "C" int tw_layer_end(float* x, const float* y, const float* w, float eps,
   layer_end_kernel<<<dim3(n, shares), 256, 0, stream>>>(x, y, w, eps, mult, history, history_stride, layer, mix, width);
   return TW_LAUNCH_RESULT();
 }
+
+// ---- token embedding plus a row of a hashed pair table, then an RMS norm -------------------------------------------
+// x[n] = w * unit(scale * table[token n] + pairs[r(n)]),  r = (previous token * mul_prev + token * mul_cur) mod
+// buckets, and r = buckets (the table's last row) for a sequence's first token. The token before a step's first
+// token of a sequence is part of the request's state: int32 [requests][2], copy `phase` read, the other copy
+// written by the block of the sequence's last token (so no block reads what another block of the launch writes).
+// A token id -1 - k stands for feed[k]. The normed row goes to x (float32) and, rounded, to out.
+template <typename T>
+__global__ __launch_bounds__(256) void embed_hashed_kernel(
+    const int* __restrict__ ids, const int* __restrict__ feed, int n_feed, const T* __restrict__ table,
+    const T* __restrict__ pairs, const float* __restrict__ norm_w, const int* __restrict__ q_start,
+    const int* __restrict__ kv_len, const int* __restrict__ state_slots, const int* __restrict__ phase,
+    int* __restrict__ state, int n_seqs, int hidden, int vocab, long buckets, long mul_prev, long mul_cur, float scale,
+    float eps, float* __restrict__ x, T* __restrict__ out) {
+  __shared__ float lds[16];
+  const int row = blockIdx.x;
+  const int s = tw_seq_of_row(q_start, n_seqs, row);
+  const int first = q_start[s], q_len = q_start[s + 1] - first;
+  const int start = kv_len[s] - q_len;
+  const int slot = state_slots[s], ph = phase[s] & 1;
+  auto resolve = [&](int id) {
+    if (id < 0) id = (feed && -1 - id < n_feed) ? feed[-1 - id] : 0;
+    return id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+  };
+  const int token = resolve(ids[row]);
+  long pair_row = buckets;
+  if (row > first) {
+    pair_row = ((long)resolve(ids[row - 1]) * mul_prev + (long)token * mul_cur) % buckets;
+  } else if (start > 0) {
+    pair_row = ((long)state[slot * 2 + ph] * mul_prev + (long)token * mul_cur) % buckets;
+  }
+  if (row == first + q_len - 1 && threadIdx.x == 0) state[slot * 2 + (1 - ph)] = token;
+  const T* e = table + (size_t)token * hidden;
+  const T* p = pairs + (size_t)pair_row * hidden;
+  float* xr = x + (size_t)row * hidden;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < hidden; c += blockDim.x) {
+    const float v = __fmaf_rn(scale, tw_to_float(e[c]), tw_to_float(p[c]));
+    xr[c] = v;
+    ss = __fmaf_rn(v, v, ss);
+  }
+  const float total = tw_block_sum(ss, lds);
+  const float rinv = 1.f / sqrtf(total / (float)hidden + eps);
+  for (int c = threadIdx.x; c < hidden; c += blockDim.x) {
+    const float r = xr[c] * rinv * norm_w[c];
+    xr[c] = r;
+    if (out) out[(size_t)row * hidden + c] = tw_from_float<T>(r);
+  }
+}
+
+extern "C" int tw_embed_hashed(int dtype, const int* ids, const int* feed, int n_feed, const void* table,
+                               const void* pairs, const float* norm_w, const int* q_start, const int* kv_len,
+                               const int* state_slots, const int* phase, int* state, int n, int n_seqs, int hidden,
+                               int vocab, long buckets, long mul_prev, long mul_cur, float scale, float eps, float* x,
+                               void* out, hipStream_t stream) {
+  TW_REQUIRE(ids && table && pairs && norm_w && q_start && kv_len && state_slots && phase && state && x);
+  TW_REQUIRE(n >= 0 && n_seqs > 0 && hidden > 0 && vocab > 0 && buckets > 0 && mul_prev >= 0 && mul_cur >= 0 && eps > 0.f);
+  if (n == 0) return 0;
+  if (dtype == TW_DTYPE_BF16)
+    embed_hashed_kernel<bf16_t><<<n, 256, 0, stream>>>(ids, feed, n_feed, (const bf16_t*)table, (const bf16_t*)pairs, norm_w,
+                                                       q_start, kv_len, state_slots, phase, state, n_seqs, hidden, vocab,
+                                                       buckets, mul_prev, mul_cur, scale, eps, x, (bf16_t*)out);
+  else if (dtype == TW_DTYPE_F32)
+    embed_hashed_kernel<float><<<n, 256, 0, stream>>>(ids, feed, n_feed, (const float*)table, (const float*)pairs, norm_w,
+                                                      q_start, kv_len, state_slots, phase, state, n_seqs, hidden, vocab,
+                                                      buckets, mul_prev, mul_cur, scale, eps, x, (float*)out);
+  else return TW_ERR_BAD_ARGUMENT;
+  return TW_LAUNCH_RESULT();
+}

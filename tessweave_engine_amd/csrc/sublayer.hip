@@ -1,0 +1,155 @@
+// Kernels of a layer arrangement that norms AFTER each sum:
+//
+//   x <- w * unit(alpha * x + scale * y),  unit(v) = v / sqrt(mean(v^2) + eps)
+//
+// x is the float32 residual stream, y a sublayer's float32 result (or split-K partial sums that are added up
+// here, in index order), scale an optional per-channel factor, w the norm's weight. The normed row is written
+// back to x and, rounded once, to `out` in the compute type, which is what the next sublayer's products read.
+// Also here: the square of relu, in place, for a feed-forward without a gate.
+#include "tw_common.h"
+
+struct ResidualNormArgs {
+  float* x;                 // [n][hidden]
+  const float* y; long ldy; // [n][ldy] or null
+  const float* add; int splits; size_t add_stride;   // [splits][n][hidden] or null
+  const float* scale;       // [hidden] or null
+  const float* w;           // [hidden]
+  void* out;                // [n][hidden], compute type, or null
+  int hidden;
+  float alpha, eps;
+};
+
+// PER groups of four consecutive elements a thread, the row in registers between the two passes.
+template <typename T, int PER>
+__global__ __launch_bounds__(1024) void residual_norm_vec4_kernel(ResidualNormArgs a) {
+  __shared__ float lds[16];
+  const int row = blockIdx.x;
+  const int chunks = a.hidden / 4;
+  float* x = a.x + (size_t)row * a.hidden;
+  f32x4 v[PER];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int c = threadIdx.x + i * blockDim.x;
+    v[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (c < chunks) {
+      f32x4 yv = {0.f, 0.f, 0.f, 0.f};
+      if (a.add) {
+        for (int s = 0; s < a.splits; ++s)
+          yv += *reinterpret_cast<const f32x4*>(a.add + s * a.add_stride + (size_t)row * a.hidden + 4 * c);
+      } else if (a.y) {
+        yv = *reinterpret_cast<const f32x4*>(a.y + (size_t)row * a.ldy + 4 * c);
+      }
+      if (a.scale) yv *= *reinterpret_cast<const f32x4*>(a.scale + 4 * c);
+      const f32x4 xv = *reinterpret_cast<const f32x4*>(x + 4 * c);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        v[i][e] = __fmaf_rn(a.alpha, xv[e], yv[e]);
+        ss = __fmaf_rn(v[i][e], v[i][e], ss);
+      }
+    }
+  }
+  const float total = tw_block_sum(ss, lds);
+  const float rinv = 1.f / sqrtf(total / (float)a.hidden + a.eps);
+  T* out = a.out ? (T*)a.out + (size_t)row * a.hidden : nullptr;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int c = threadIdx.x + i * blockDim.x;
+    if (c < chunks) {
+      const f32x4 wv = *reinterpret_cast<const f32x4*>(a.w + 4 * c);
+      f32x4 r;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) r[e] = v[i][e] * rinv * wv[e];
+      *reinterpret_cast<f32x4*>(x + 4 * c) = r;
+      if (out) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) out[4 * c + e] = tw_from_float<T>(r[e]);
+      }
+    }
+  }
+}
+
+// Any row length: the sums are parked in x between the two passes (a thread reads back only what it wrote).
+template <typename T>
+__global__ void residual_norm_kernel(ResidualNormArgs a) {
+  __shared__ float lds[16];
+  const int row = blockIdx.x;
+  float* x = a.x + (size_t)row * a.hidden;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < a.hidden; c += blockDim.x) {
+    float yv = 0.f;
+    if (a.add) {
+      for (int s = 0; s < a.splits; ++s) yv += a.add[s * a.add_stride + (size_t)row * a.hidden + c];
+    } else if (a.y) {
+      yv = a.y[(size_t)row * a.ldy + c];
+    }
+    if (a.scale) yv *= a.scale[c];
+    const float v = __fmaf_rn(a.alpha, x[c], yv);
+    x[c] = v;
+    ss = __fmaf_rn(v, v, ss);
+  }
+  const float total = tw_block_sum(ss, lds);
+  const float rinv = 1.f / sqrtf(total / (float)a.hidden + a.eps);
+  T* out = a.out ? (T*)a.out + (size_t)row * a.hidden : nullptr;
+  for (int c = threadIdx.x; c < a.hidden; c += blockDim.x) {
+    const float r = x[c] * rinv * a.w[c];
+    x[c] = r;
+    if (out) out[c] = tw_from_float<T>(r);
+  }
+}
+
+template <typename T>
+static void residual_norm_launch(const ResidualNormArgs& a, int n, hipStream_t stream) {
+  const bool aligned = a.hidden % 4 == 0 && (uintptr_t)a.x % 16 == 0 && (uintptr_t)a.w % 16 == 0 &&
+                       (!a.y || ((uintptr_t)a.y % 16 == 0 && a.ldy % 4 == 0)) &&
+                       (!a.add || ((uintptr_t)a.add % 16 == 0 && a.add_stride % 4 == 0)) &&
+                       (!a.scale || (uintptr_t)a.scale % 16 == 0);
+  const int chunks = a.hidden / 4;
+  if (aligned && chunks <= 4096) {
+    const int per = chunks <= 1024 ? 1 : (chunks <= 2048 ? 2 : 4);
+    int threads = (chunks + per - 1) / per;
+    threads = (threads + 63) / 64 * 64;
+    if (per == 1) residual_norm_vec4_kernel<T, 1><<<n, threads, 0, stream>>>(a);
+    else if (per == 2) residual_norm_vec4_kernel<T, 2><<<n, threads, 0, stream>>>(a);
+    else residual_norm_vec4_kernel<T, 4><<<n, threads, 0, stream>>>(a);
+  } else {
+    residual_norm_kernel<T><<<n, 256, 0, stream>>>(a);
+  }
+}
+
+extern "C" int tw_residual_norm(int out_dtype, float* x, const float* y, long ldy, const float* add, int splits,
+                                long add_stride, const float* scale, const float* w, void* out, int n, int hidden,
+                                float alpha, float eps, hipStream_t stream) {
+  TW_REQUIRE(x && w && n >= 0 && hidden > 0 && eps > 0.f);
+  TW_REQUIRE(add == nullptr || (splits > 0 && add_stride >= (long)n * hidden));
+  TW_REQUIRE(y == nullptr || ldy >= hidden);
+  if (n == 0) return 0;
+  ResidualNormArgs a{x, add ? nullptr : y, ldy, add, splits, (size_t)add_stride, scale, w, out, hidden, alpha, eps};
+  if (out_dtype == TW_DTYPE_BF16) residual_norm_launch<bf16_t>(a, n, stream);
+  else if (out_dtype == TW_DTYPE_F32) residual_norm_launch<float>(a, n, stream);
+  else return TW_ERR_BAD_ARGUMENT;
+  return TW_LAUNCH_RESULT();
+}
+
+// ---- x <- max(x, 0)^2 in place ---------------------------------------------------------------------------
+template <typename T>
+__global__ void relu_squared_kernel(T* __restrict__ x, long ld, int cols, long total) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const long row = i / cols;
+  const int col = (int)(i % cols);
+  T* p = x + row * ld + col;
+  const float v = fmaxf(tw_to_float(*p), 0.f);
+  *p = tw_from_float<T>(v * v);
+}
+
+extern "C" int tw_relu_squared(int dtype, void* x, long ld, int n, int cols, hipStream_t stream) {
+  TW_REQUIRE(x && n >= 0 && cols > 0 && ld >= cols);
+  if (n == 0) return 0;
+  const long total = (long)n * cols;
+  const int blocks = tw_div_up(total, 256);
+  if (dtype == TW_DTYPE_BF16) relu_squared_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)x, ld, cols, total);
+  else if (dtype == TW_DTYPE_F32) relu_squared_kernel<float><<<blocks, 256, 0, stream>>>((float*)x, ld, cols, total);
+  else return TW_ERR_BAD_ARGUMENT;
+  return TW_LAUNCH_RESULT();
+}

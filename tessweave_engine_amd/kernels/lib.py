@@ -21,7 +21,7 @@ _SIGNATURES = {
     "tw_upload_words": (I, [P, P, I, ctypes.POINTER(c_int), ctypes.POINTER(c_int), P]),
     "tw_embed_gather": (I, [I, P, P, P, I, I, I, P, I, P]),
     "tw_rmsnorm": (I, [I, P, P, P, P, I, I, F, P, I, L, P, P]),
-    "tw_rope_table": (I, [P, P, P, P, I, I, P]),
+    "tw_rope_table": (I, [P, P, P, P, I, I, F, P]),
     "tw_rope_kv_write": (I, [I, P, L, P, P, P, P, P, I, I, I, I, I, I, I, P, I, P, I, P]),
     "tw_silu_mul": (I, [I, P, P, I, I, P]),
     "tw_linear_workspace_bytes": (L, [I, I, I, I]),
@@ -50,6 +50,13 @@ _SIGNATURES = {
     "tw_attn_mixed_workspace_floats": (L, [I, I, I, I, I]),
     "tw_attn_mixed": (I, [I, P, L, P, P, P, I, P, P, I, I, I, P, L, P, P, P, P, L, I, I, I, I, I, I, F, F, I, P]),
     "tw_kv_store": (I, [I, P, L, I, I, P, P, P, I, I, I, I, I, P]),
+    "tw_residual_norm": (I, [I, P, P, L, P, I, L, P, P, P, I, I, F, F, P]),
+    "tw_relu_squared": (I, [I, P, L, I, I, P]),
+    "tw_embed_hashed": (I, [I, P, P, I, P, P, P, P, P, P, P, P, I, I, I, I, L, L, L, F, F, P, P, P]),
+    "tw_latent_finish": (I, [I, P, L, I, I, I, P, P, P, P, L, P, P, P, I, I, I, I, I, I, I, F, P]),
+    "tw_head_linear": (I, [I, P, L, I, P, P, L, I, I, I, I, I, P]),
+    "tw_retention": (I, [I, P, L, I, I, I, P, P, I, P, P, P, P, P, L, I, I, I, I, I, F, P]),
+    "tw_unit_gate": (I, [I, P, L, P, L, P, L, I, I, I, I, F, P]),
     "tw_sampling_uniform": (F, [c_uint64, c_uint64]),
     "tw_sample_workspace_bytes": (L, [I]),
     "tw_sample_rows": (I, [P, L, I, I, P, P, P, P, P, L, P]),

@@ -115,15 +115,15 @@ def rmsnorm(x, weight, eps, out, rows=None, add=None, row_scratch=None):
     return out
 
 
-def rope_table(positions, inv_freq, cos, sin):
-    """cos/sin[n, j] of float32(positions[n]) * inv_freq[j]."""
+def rope_table(positions, inv_freq, cos, sin, magnitude=1.0):
+    """cos/sin[n, j] of float32(positions[n]) * inv_freq[j], both times MAGNITUDE."""
     n, half = positions.numel(), inv_freq.numel()
     _need(cos.is_contiguous() and sin.is_contiguous() and tuple(cos.shape) == (n, half)
           and tuple(sin.shape) == (n, half), "rotary tables must be [n, rot/2]")
     check(library().tw_rope_table(_dev(positions, torch.int32, "positions"),
                                   _dev(inv_freq, torch.float32, "inv_freq"),
                                   _dev(cos, torch.float32, "cos"), _dev(sin, torch.float32, "sin"),
-                                  n, half, _stream()), "rope_table")
+                                  n, half, float(magnitude), _stream()), "rope_table")
 
 
 def rope_kv_write(qkv, cos, sin, slots, keys, values, q_heads, kv_heads, head_dim, page_size,
@@ -708,4 +708,165 @@ def attn_mixed(q, keys, values, block_table, q_start, kv_len, seq0, n_seqs, max_
                                   _dev(slopes) if slopes is not None else None, ws_ptr, ws_floats, q_heads, kv_heads,
                                   key_dim, value_dim, page, int(window or 0), float(scale), float(out_scale), int(splits),
                                   _stream()), "attn_mixed")
+    return out
+
+
+# ---- norm after the sum, relu squared, hashed pair embedding ----------------------------------------------------------
+
+def residual_norm(x, weight, eps, out=None, y=None, add=None, scale=None, alpha=1.0):
+    """x <- weight * unit(alpha * x + scale * y), unit(v) = v / sqrt(mean(v^2) + eps); x float32 [n, hidden] in place.
+
+    y: float32 [n, hidden] (rows may be strided), or add: float32 [splits, n, hidden] partial sums added up here;
+    scale: float32 [hidden] or None; out: the normed rows once more, rounded to its type (the compute type)."""
+    _need(x.dim() == 2 and x.is_contiguous() and x.dtype == torch.float32, "residual_norm: x must be contiguous float32 [n, hidden]")
+    n, hidden = x.shape
+    _need(weight.numel() == hidden and weight.dtype == torch.float32 and weight.is_contiguous(), "the norm weight must be float32 [hidden]")
+    ldy = 0
+    if y is not None:
+        ny, cy, ldy = _rows(y, "y")
+        _need((ny, cy) == (n, hidden) and y.dtype == torch.float32, "y must be float32 [n, hidden]")
+    splits, stride = 0, 0
+    if add is not None:
+        _need(y is None, "either y or partial sums")
+        _need(add.dim() == 3 and add.is_contiguous() and tuple(add.shape[1:]) == (n, hidden) and add.dtype == torch.float32,
+              "partial sums must be float32 [splits, n, hidden]")
+        splits, stride = add.shape[0], n * hidden
+    if scale is not None:
+        _need(scale.numel() == hidden and scale.dtype == torch.float32 and scale.is_contiguous(), "scale must be float32 [hidden]")
+    out_dtype = F32
+    if out is not None:
+        _need(out.is_contiguous() and tuple(out.shape) == (n, hidden), "out must be contiguous [n, hidden]")
+        out_dtype = dtype_id(out.dtype)
+    check(library().tw_residual_norm(out_dtype, _dev(x), _dev(y) if y is not None else None, ldy,
+                                     _dev(add) if add is not None else None, splits, stride,
+                                     _dev(scale) if scale is not None else None, _dev(weight),
+                                     _dev(out) if out is not None else None, n, hidden, float(alpha), float(eps), _stream()),
+          "residual_norm")
+    return x
+
+
+def relu_squared(x):
+    """x <- max(x, 0)^2 in place (rows may be strided)."""
+    n, cols, ld = _rows(x, "x")
+    check(library().tw_relu_squared(dtype_id(x.dtype), _dev(x), ld, n, cols, _stream()), "relu_squared")
+    return x
+
+
+def embed_hashed(ids, table, pairs, norm_weight, q_start, kv_len, state_slots, phase, state, n_seqs, buckets, mul_prev,
+                 mul_cur, scale, eps, x, out=None, feed=None):
+    """x[n] = norm_weight * unit(scale * table[ids[n]] + pairs[r]), r = (previous token * mul_prev + token * mul_cur) mod
+    buckets, r = buckets for a sequence's first token. state int32 [requests, 2] holds the last token of every request
+    twice (copy phase[s] is read, the other written). x float32 [n, hidden]; out: the same rounded to its type."""
+    n = ids.numel()
+    vocab, hidden = table.shape
+    _need(table.is_contiguous() and pairs.is_contiguous() and pairs.dtype == table.dtype and tuple(pairs.shape) == (buckets + 1, hidden),
+          "the pair table must be [buckets + 1, hidden] of the embedding's type")
+    _need(x.is_contiguous() and tuple(x.shape) == (n, hidden) and x.dtype == torch.float32, "x must be float32 [n, hidden]")
+    _need(norm_weight.numel() == hidden and norm_weight.dtype == torch.float32, "the norm weight must be float32 [hidden]")
+    _need(state.dtype == torch.int32 and state.is_contiguous() and state.dim() == 2 and state.shape[1] == 2, "state must be int32 [requests, 2]")
+    _need(q_start.numel() >= n_seqs + 1 and kv_len.numel() >= n_seqs and state_slots.numel() >= n_seqs and phase.numel() >= n_seqs,
+          "sequence metadata is too short")
+    if out is not None:
+        _need(out.is_contiguous() and tuple(out.shape) == (n, hidden) and out.dtype == table.dtype, "out must be [n, hidden] of the table's type")
+    check(library().tw_embed_hashed(dtype_id(table.dtype), _dev(ids, torch.int32, "ids"),
+                                    _dev(feed, torch.int32, "feed") if feed is not None else None,
+                                    feed.numel() if feed is not None else 0, _dev(table), _dev(pairs), _dev(norm_weight),
+                                    _dev(q_start, torch.int32, "q_start"), _dev(kv_len, torch.int32, "kv_len"),
+                                    _dev(state_slots, torch.int32, "state_slots"), _dev(phase, torch.int32, "phase"),
+                                    _dev(state), n, int(n_seqs), hidden, vocab, int(buckets), int(mul_prev), int(mul_cur),
+                                    float(scale), float(eps), _dev(x), _dev(out) if out is not None else None, _stream()),
+          "embed_hashed")
+    return x
+
+
+# ---- attention over a cached latent: finishing a token's projections, one small matrix per head -----------------------
+
+def latent_finish(proj, q_col, c_col, kr_col, cos, sin, norm_weight, q_out, heads, latent, latent_dev, rot_dev, eps,
+                  keys=None, values=None, slots=None):
+    """Rotates the heads' rotated query parts proj[n, q_col + a * rot_dev ...] into q_out[n, a, latent_dev:], and,
+    with keys/values, stores the token's key row [unit(proj[n, c_col : c_col + latent]) * norm_weight | zeros |
+    rotated proj[n, kr_col ...] | zeros] and its value (the normed latent) into page slot slots[n] (-1: not stored).
+    keys [pages, 1, page, latent_dev + rot_dev]; values [pages, 1, latent_dev, page]; q_out [n, heads * (latent_dev + rot_dev)]."""
+    n, width, ld = _rows(proj, "proj")
+    rot = 2 * cos.shape[1]
+    _need(tuple(cos.shape) == (n, rot // 2) and tuple(sin.shape) == (n, rot // 2) and cos.is_contiguous() and sin.is_contiguous()
+          and cos.dtype == torch.float32, "rotary tables must be float32 [n, rot / 2]")
+    nq, wq, ldq = _rows(q_out, "q_out")
+    K = latent_dev + rot_dev
+    _need(nq == n and wq == heads * K and q_out.dtype == proj.dtype, "q_out must be [n, heads * (latent_dev + rot_dev)] of proj's type")
+    _need(q_col + heads * rot_dev <= width and rot <= rot_dev, "the rotated query parts exceed the projection's row")
+    page = 0
+    if keys is not None:
+        page = keys.shape[2]
+        _need(keys.is_contiguous() and values.is_contiguous() and keys.dtype == proj.dtype == values.dtype, "cache and projection types differ")
+        _need(tuple(keys.shape[1:]) == (1, page, K) and tuple(values.shape) == (keys.shape[0], 1, latent_dev, page),
+              "keys [pages, 1, page, latent_dev + rot_dev], values [pages, 1, latent_dev, page]")
+        _need(slots.numel() == n and norm_weight.numel() == latent and norm_weight.dtype == torch.float32 and latent <= latent_dev,
+              "one slot per token and a float32 norm weight per latent element are needed")
+        _need(c_col + latent <= width and kr_col + rot <= width, "the latent or the shared key part exceed the projection's row")
+    check(library().tw_latent_finish(dtype_id(proj.dtype), _dev(proj), ld, int(q_col), int(c_col), int(kr_col), _dev(cos), _dev(sin),
+                                     _dev(norm_weight) if keys is not None else None, _dev(q_out), ldq,
+                                     _dev(keys) if keys is not None else None, _dev(values) if keys is not None else None,
+                                     _dev(slots, torch.int32, "slots") if keys is not None else None, n, heads, int(latent),
+                                     int(latent_dev), int(rot_dev), rot, page, float(eps), _stream()), "latent_finish")
+
+
+def head_linear(x, x_stride, weight, out, out_stride):
+    """out[n, a * out_stride + o] = sum_i x[n, a * x_stride + i] * weight[a, o, i]; weight [heads, No, Ni] of x's type
+    (Ni a multiple of 16 bytes, No of 4); out has x's type; float32 sums, one rounding."""
+    n, wx, ldx = _rows(x, "x")
+    no, wo, ldo = _rows(out, "out")
+    heads, n_out, n_in = weight.shape
+    epf = 16 // x.element_size()
+    _need(weight.is_contiguous() and weight.dtype == x.dtype == out.dtype and no == n, "head_linear operand types or rows differ")
+    _need(n_in % epf == 0 and n_out % 4 == 0 and x_stride % epf == 0 and ldx % epf == 0 and x.data_ptr() % 16 == 0,
+          "head_linear: inputs must be 16-byte aligned and Ni a multiple of 16 bytes, No of 4")
+    _need((heads - 1) * x_stride + n_in <= wx and (heads - 1) * out_stride + n_out <= wo and out_stride >= n_out,
+          "head_linear: the heads exceed the rows")
+    _need((ldo * out.element_size()) % 8 == 0 and (out_stride * out.element_size()) % 8 == 0 and out.data_ptr() % 8 == 0,
+          "head_linear: output rows and heads must be 8-byte aligned")
+    check(library().tw_head_linear(dtype_id(x.dtype), _dev(x), ldx, int(x_stride), _dev(weight), _dev(out), ldo, int(out_stride),
+                                   n, heads, n_in, n_out, _stream()), "head_linear")
+    return out
+
+
+# ---- retention ------------------------------------------------------------------------------------------------
+
+def retention(proj, q_col, k_col, v_col, cos, sin, decay, state, q_start, state_slots, n_seqs, max_q_len, out, k_scale):
+    """S_t = decay_h S_(t-1) + k_t v_t^T, o_t = S_t^T q_t per sequence and head, from and to state float32
+    [requests, H, Dp, Ep]. q, k (unrotated) and v are columns of proj (head h at col + h * Dp, or + h * Ep); they are
+    rotated with cos/sin float32 [n, rot / 2] (None: no rotation) and k then multiplied by k_scale. out float32
+    [n, H * Ep]."""
+    n, width, ld = _rows(proj, "proj")
+    _need(state.dim() == 4 and state.is_contiguous() and state.dtype == torch.float32, "state must be float32 [requests, H, Dp, Ep]")
+    H, Dp, Ep = state.shape[1:]
+    rot = 0
+    if cos is not None:
+        rot = 2 * cos.shape[1]
+        _need(tuple(cos.shape) == (n, rot // 2) and tuple(sin.shape) == (n, rot // 2) and cos.is_contiguous() and sin.is_contiguous()
+              and cos.dtype == torch.float32, "rotary tables must be float32 [n, rot / 2]")
+    _need(Dp % 16 == 0 and Dp <= 256 and rot <= Dp, "key heads are multiples of 16 up to 256 on the device")
+    _need(max(q_col, k_col) + H * Dp <= width and v_col + H * Ep <= width, "q, k or v exceed the projection's row")
+    no, wo, ldo = _rows(out, "out")
+    _need(no == n and wo == H * Ep and out.dtype == torch.float32, "out must be float32 [n, H * Ep]")
+    _need(decay.numel() == H and decay.dtype == torch.float32, "one float32 decay per head")
+    _need(q_start.numel() >= n_seqs + 1 and state_slots.numel() >= n_seqs, "sequence metadata is too short")
+    check(library().tw_retention(dtype_id(proj.dtype), _dev(proj), ld, int(q_col), int(k_col), int(v_col),
+                                 _dev(cos) if rot else None, _dev(sin) if rot else None, rot, _dev(decay), _dev(state),
+                                 _dev(q_start, torch.int32, "q_start"), _dev(state_slots, torch.int32, "state_slots"),
+                                 _dev(out), ldo, int(n_seqs), max(1, int(max_q_len)), H, Dp, Ep, float(k_scale), _stream()),
+          "retention")
+    return out
+
+
+def unit_gate(o, gate, out, heads, value_dim, value_dev, eps):
+    """out[n, h, e] = o[n, h, e] / sqrt(mean_e o^2 + eps) * silu(gate[n, h, e]) over each head's value_dim real
+    elements (heads value_dev apart, tails zero); o float32, gate and out of the compute type."""
+    n, wo, ld_o = _rows(o, "o")
+    ng, wg, ld_g = _rows(gate, "gate")
+    nn, wn, ld_n = _rows(out, "out")
+    _need(o.dtype == torch.float32 and gate.dtype == out.dtype, "o is float32; gate and out share the compute type")
+    _need(ng == n and nn == n and min(wo, wg, wn) >= heads * value_dev and value_dim <= value_dev, "unit_gate shapes do not agree")
+    check(library().tw_unit_gate(dtype_id(out.dtype), _dev(o), ld_o, _dev(gate), ld_g, _dev(out), ld_n, n, heads, int(value_dim),
+                                 int(value_dev), float(eps), _stream()), "unit_gate")
     return out

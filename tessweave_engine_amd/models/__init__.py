@@ -1,3 +1,4 @@
 """Built-in architectures; importing this package registers them."""
 from . import qwen2  # noqa: F401
 from . import kanavik  # noqa: F401
+from . import dinutar  # noqa: F401

@@ -4,12 +4,14 @@ from .linear import JoinedLinear, Linear
 from .norms import RMSNorm
 from .positions import NoPositionEncoding, RotaryEmbedding
 from .attention import GroupedQueryAttention
-from .feedforward import GatedFeedForward, SwiGLU
-from .blocks import DepthMixedBlock, PreNormBlock
-from .embedding import OutputHead, PositionedEmbedding, TokenEmbedding
+from .feedforward import GatedFeedForward, ReluSquaredFeedForward, SwiGLU
+from .blocks import DepthMixedBlock, PostNormBlock, PreNormBlock
+from .embedding import HashedPairEmbedding, OutputHead, PositionedEmbedding, TokenEmbedding
 from .convolution import CausalConv
 from .parallel import GatedLinearRecurrence, MixedHeadAttention, MixerBranch, ParallelMixer
 from .side_input import SideTable, TokenSideInput
+from .latent import LatentAttention
+from .retention import Retention
 from .model import DecoderModel, walk
 
 __all__ = ["Block", "FeedForward", "GroupStep", "HeadHook", "LayerRun", "Mixer", "Norm", "Part", "PositionEncoding",
@@ -17,4 +19,5 @@ __all__ = ["Block", "FeedForward", "GroupStep", "HeadHook", "LayerRun", "Mixer",
            "GroupedQueryAttention", "SwiGLU", "PreNormBlock", "OutputHead", "TokenEmbedding",
            "JoinedLinear", "GatedFeedForward", "DepthMixedBlock", "PositionedEmbedding", "CausalConv",
            "GatedLinearRecurrence", "MixedHeadAttention", "MixerBranch", "ParallelMixer", "SideTable", "TokenSideInput",
+           "HashedPairEmbedding", "LatentAttention", "PostNormBlock", "ReluSquaredFeedForward", "Retention",
            "DecoderModel", "walk"]

@@ -67,7 +67,7 @@ class GroupedQueryAttention(Mixer):
     def cache_need(self):
         return CacheNeed(paged=PagedKV(self.kv_heads, self.head_dim, self.window))
 
-    def forward(self, ctx, run, h, x):
+    def forward(self, ctx, run, h, x, accumulate=True):
         n = ctx.n_tokens
         width = (self.q_heads + 2 * self.kv_heads) * self.head_dim
         qkv = ctx.scratch("attn.qkv", (n, width))
@@ -121,5 +121,5 @@ class GroupedQueryAttention(Mixer):
                              softcap=self.softcap)
         if ctx.defer_sums and not self.o.biases and self.o.deferrable(n):
             return self.o.forward_partials(ctx, out, "o")          # the next norm adds them into x
-        self.o.forward(ctx, out, x, residual=x)
+        self.o.forward(ctx, out, x, residual=x if accumulate else None)
         return None

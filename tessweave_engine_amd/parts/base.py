@@ -16,6 +16,11 @@ import math
 import torch
 
 
+#: key of `StepContext.shared` under which a part that has just written the residual stream may leave the same rows
+#: rounded to the compute type (in float32 runs: the stream itself), for a sublayer that reads the stream as it is
+ROUNDED_STREAM = "stream.rounded"
+
+
 @dataclass(frozen=True)
 class LayerRun:
     """One entry of a model's schedule.
@@ -106,6 +111,10 @@ class Mixer(Part):
 
     def forward(self, ctx, run, h, x):
         """Add the mixer's output for normalised input H into the residual stream X (float32, in place).
+
+        Mixers that an arrangement may ask for their result ALONE (one that scales it or norms the sum) take a
+        further keyword `accumulate`: with accumulate=False the result is written to X (any float32 [n, hidden]
+        buffer) instead of added, or returned as pending partial sums of the result alone.
 
         Returns None, or, only if `ctx.defer_sums` allows it, PENDING partial sums (float32
         [splits, n, hidden]) that are not yet in X: whoever runs next (the following norm) adds them up

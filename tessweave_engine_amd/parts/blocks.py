@@ -8,8 +8,8 @@ import torch
 
 from ..cache.spec import CacheNeed
 from ..kernels import ops
-from ..weights.spec import AVERAGE, VECTOR, TensorSpec
-from .base import Block, fold_pending
+from ..weights.spec import AVERAGE, ONE_PLUS_NORMAL, VECTOR, TensorSpec
+from .base import ROUNDED_STREAM, Block, fold_pending
 
 
 class PreNormBlock(Block):
@@ -41,6 +41,73 @@ def normalise(norm, ctx, x, pending=None, rows=None):
     if pending is not None:
         return norm.forward(ctx, x, rows=rows, add=pending)
     return norm.forward(ctx, x, rows=rows)
+
+
+class PostNormBlock(Block):
+    """Norm after the sum, with an optional scale per channel on each sublayer's result:
+
+        x <- norm1(alpha * x + scale1 * mixer(x));  x <- norm2(alpha * x + scale2 * ff(x))
+
+    The sublayers read the stream x itself (rounded to the compute type). mixer_norm, ffn_norm: `RMSNorm` parts
+    (weight and eps; sum, scale, norm and the rounding for the next sublayer are one kernel, which also adds up
+    split-K partial sums a sublayer leaves pending). ffn / ffn_norm may be None: the layer then has only the
+    first sublayer. scale names: float32 [hidden] checkpoint tensors, or None. The mixer and the feed-forward
+    must take `accumulate=False` (their result alone, not added into the stream)."""
+
+    def __init__(self, hidden, mixer, mixer_norm, ffn=None, ffn_norm=None, alpha=1.0, mixer_scale_name=None,
+                 ffn_scale_name=None):
+        if (ffn is None) != (ffn_norm is None):
+            raise ValueError("a feed-forward and its norm come together")
+        self.hidden, self.alpha = int(hidden), float(alpha)
+        self.mixer, self.mixer_norm, self.ffn, self.ffn_norm = mixer, mixer_norm, ffn, ffn_norm
+        self.mixer_scale_name = mixer_scale_name
+        self.ffn_scale_name = ffn_scale_name if ffn is not None else None
+        self.mixer_scale = self.ffn_scale = None
+
+    def parts(self):
+        return [p for p in (self.mixer, self.mixer_norm, self.ffn, self.ffn_norm) if p is not None]
+
+    def tensor_specs(self):
+        specs = [s for p in self.parts() for s in p.tensor_specs()]
+        for name in (self.mixer_scale_name, self.ffn_scale_name):
+            if name:
+                specs.append(TensorSpec(name, (self.hidden,), VECTOR, ONE_PLUS_NORMAL))
+        return specs
+
+    def bind(self, tensors, dtype, device):
+        for p in self.parts():
+            p.bind(tensors, dtype, device)
+        self.mixer_scale = tensors.pop(self.mixer_scale_name).contiguous() if self.mixer_scale_name else None
+        self.ffn_scale = tensors.pop(self.ffn_scale_name).contiguous() if self.ffn_scale_name else None
+
+    def weight_tensors(self):
+        return [t for t in (self.mixer_scale, self.ffn_scale) if t is not None]
+
+    def _rounded(self, ctx, x):
+        """The stream in the compute type: what the part before left, else rounded now (float32 runs read x itself)."""
+        h = ctx.shared.get(ROUNDED_STREAM)
+        if h is None:
+            if ctx.dtype == torch.float32:
+                return x
+            h = ops.round_rows(x, ctx.scratch("stream.rounded", (ctx.n_tokens, self.hidden)))
+        return h
+
+    def _sublayer(self, ctx, x, norm, scale, result, pending):
+        rounded = ctx.scratch("stream.rounded", (ctx.n_tokens, self.hidden)) if ctx.dtype != torch.float32 else None
+        ops.residual_norm(x, norm.weight, norm.eps, out=rounded, y=result if pending is None else None, add=pending,
+                          scale=scale, alpha=self.alpha)
+        ctx.shared[ROUNDED_STREAM] = rounded if rounded is not None else x
+
+    def forward(self, ctx, run, x, pending=None):
+        pending = fold_pending(x, pending)
+        n = ctx.n_tokens
+        result = ctx.scratch("sublayer.result", (n, self.hidden), torch.float32)
+        left = self.mixer.forward(ctx, run, self._rounded(ctx, x), result, accumulate=False)
+        self._sublayer(ctx, x, self.mixer_norm, self.mixer_scale, result, left)
+        if self.ffn is not None:
+            left = self.ffn.forward(ctx, self._rounded(ctx, x), result, accumulate=False)
+            self._sublayer(ctx, x, self.ffn_norm, self.ffn_scale, result, left)
+        return None
 
 
 class DepthMixedBlock(Block):

@@ -9,9 +9,10 @@ from __future__ import annotations
 
 import torch
 
+from ..cache.spec import CacheNeed, FixedState
 from ..kernels import ops
 from ..weights.spec import MATRIX, NORMAL, TensorSpec
-from .base import Part
+from .base import ROUNDED_STREAM, Part
 
 
 class TokenEmbedding(Part):
@@ -58,6 +59,58 @@ class PositionedEmbedding(TokenEmbedding):
             tag, leading = self.keep
             copy = ctx.workspace.get(tag, (leading, ctx.max_tokens, self.hidden), torch.float32)[0, :ctx.n_tokens]
         return ops.add_table_rows(x, self.positions, ctx.positions[0], copy=copy)
+
+
+class HashedPairEmbedding(TokenEmbedding):
+    """Token embedding times a scale, plus a row of a table indexed by a hash of (previous token, token), then a norm:
+
+        x = norm( scale * table[token] + pairs[(previous * mul_prev + token * mul_cur) mod buckets] )
+
+    A sequence's first token has no previous one and takes the pair table's last row (number `buckets`). The
+    last token of a request is part of its state (`cache_need`: an int32 state in a cache slot of the part's
+    own, which the model assigns), so a prompt cut into portions and a decoded token find their predecessor
+    there. The state is held twice, as every state that one block of a launch reads and another writes. norm: an
+    `RMSNorm` part (its weight and eps are used; embedding, sum and norm are one kernel). The normed row is left in
+    the float32 residual stream and, rounded to the compute type, under `ctx.shared[ROUNDED_STREAM]`."""
+
+    STATE = "last_token"
+
+    def __init__(self, name, vocab, hidden, pair_name, buckets, mul_prev, mul_cur, norm, scale=1.0, suffix=".weight"):
+        super().__init__(name, vocab, hidden, suffix)
+        self.pair_name, self.buckets = pair_name, int(buckets)
+        self.mul_prev, self.mul_cur, self.scale, self.norm = int(mul_prev), int(mul_cur), float(scale), norm
+        if self.buckets <= 0 or self.mul_prev < 0 or self.mul_cur < 0:
+            raise ValueError("buckets must be positive and the multipliers not negative")
+        self.pairs = None
+        self.cache_slot = None            # set by the model when it lays its cache out
+
+    def parts(self):
+        return [self.norm]
+
+    def tensor_specs(self):
+        return (super().tensor_specs() + [TensorSpec(self.pair_name + self.suffix, (self.buckets + 1, self.hidden), MATRIX, NORMAL)]
+                + self.norm.tensor_specs())
+
+    def bind(self, tensors, dtype, device):
+        super().bind(tensors, dtype, device)
+        self.pairs = tensors.pop(self.pair_name + self.suffix).contiguous()
+        self.norm.bind(tensors, dtype, device)
+
+    def cache_need(self):
+        return CacheNeed(states=((self.STATE, FixedState((2,), "int32")),))
+
+    def forward(self, ctx):
+        if self.cache_slot is None:
+            raise RuntimeError("the model has not given this embedding a cache slot (its cache layout was never asked for)")
+        n = ctx.n_tokens
+        x = ctx.scratch("residual", (n, self.hidden), torch.float32)
+        rounded = ctx.scratch("stream.rounded", (n, self.hidden)) if ctx.dtype != torch.float32 else None
+        state = ctx.cache.states[self.cache_slot][self.STATE]
+        ops.embed_hashed(ctx.token_ids, self.weight, self.pairs, self.norm.weight, ctx.q_start, ctx.kv_len, ctx.state_slots,
+                         ctx.state_phase, state, ctx.n_seqs, self.buckets, self.mul_prev, self.mul_cur, self.scale,
+                         self.norm.eps, x, out=rounded, feed=ctx.token_feed)
+        ctx.shared[ROUNDED_STREAM] = rounded if rounded is not None else x
+        return x
 
 
 class OutputHead(Part):

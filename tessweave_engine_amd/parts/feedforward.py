@@ -1,4 +1,8 @@
-"""SwiGLU feed-forward: x += down( silu(gate(h)) * up(h) ), no biases (flow_engine/model.py:68-85)."""
+"""SwiGLU feed-forward: x += down( silu(gate(h)) * up(h) ), no biases (flow_engine/model.py:68-85); the same with
+another activation (`GatedFeedForward`); and one without a gate, down( relu(up(h))^2 ) (`ReluSquaredFeedForward`).
+
+`accumulate=False` asks for the result alone (written to x, or left as pending partial sums of the result alone),
+for arrangements that scale it or norm the sum."""
 from __future__ import annotations
 
 from ..kernels import ops
@@ -23,7 +27,7 @@ class SwiGLU(FeedForward):
         self.gate_up.bind(tensors, dtype, device)
         self.down.bind(tensors, dtype, device)
 
-    def forward(self, ctx, h, x):
+    def forward(self, ctx, h, x, accumulate=True):
         n = h.shape[0]
         act = ctx.scratch("ffn.act", (n, self.intermediate))
         if self.gate_up.gated:
@@ -36,7 +40,7 @@ class SwiGLU(FeedForward):
         if ctx.defer_sums and not self.down.biases and self.down.deferrable(n):
             # where the down projection splits K (few rows; many rows against its long K), the sums are left to the next norm
             return self.down.forward_partials(ctx, act, "down")
-        self.down.forward(ctx, act, x, residual=x)
+        self.down.forward(ctx, act, x, residual=x if accumulate else None)
         return None
 
 
@@ -69,7 +73,7 @@ class GatedFeedForward(FeedForward):
         self.gate_up.bind(tensors, dtype, device)
         self.down.bind(tensors, dtype, device)
 
-    def forward(self, ctx, h, x):
+    def forward(self, ctx, h, x, accumulate=True):
         n = h.shape[0]
         act = ctx.scratch("ffn.act", (n, self.intermediate))
         if self.gate_up.gated:
@@ -78,5 +82,35 @@ class GatedFeedForward(FeedForward):
             gu = ctx.scratch("ffn.gate_up", (n, 2 * self.intermediate))
             self.gate_up.forward(ctx, h, gu)
             ops.gelu_mul(gu, act, self.out_scale)
-        self.down.forward(ctx, act, x, residual=x)
+        self.down.forward(ctx, act, x, residual=x if accumulate else None)
+        return None
+
+
+class ReluSquaredFeedForward(FeedForward):
+    """x += down( relu(up(h))^2 ): no gate, no biases. names = (up, down), the checkpoint prefixes of the two matrices."""
+
+    def __init__(self, names, hidden, intermediate, suffix=".weight"):
+        up, down = names
+        self.hidden, self.intermediate = int(hidden), int(intermediate)
+        self.up = Linear([up], hidden, [intermediate], suffixes=(suffix, ".bias"))
+        self.down = Linear([down], intermediate, [hidden], suffixes=(suffix, ".bias"))
+
+    def parts(self):
+        return [self.up, self.down]
+
+    def tensor_specs(self):
+        return self.up.tensor_specs() + self.down.tensor_specs()
+
+    def bind(self, tensors, dtype, device):
+        self.up.bind(tensors, dtype, device)
+        self.down.bind(tensors, dtype, device)
+
+    def forward(self, ctx, h, x, accumulate=True):
+        n = h.shape[0]
+        act = ctx.scratch("ffn.act", (n, self.intermediate))
+        self.up.forward(ctx, h, act)
+        ops.relu_squared(act)
+        if ctx.defer_sums and self.down.deferrable(n):
+            return self.down.forward_partials(ctx, act, "down")          # whoever norms next adds them up
+        self.down.forward(ctx, act, x, residual=x if accumulate else None)
         return None

@@ -100,6 +100,12 @@ class DecoderModel(Part):
                 need = self.blocks[run.block].cache_need()
                 if not run.writes_cache and needs[run.cache_slot] != need:
                     raise ValueError(f"a layer reads cache slot {run.cache_slot}, which holds something else")
+            # an embedding that carries something from token to token gets a cache slot of its own behind the layers'
+            own = getattr(self.embedding, "cache_need", None)
+            need = own() if own is not None else None
+            if need is not None:
+                self.embedding.cache_slot = len(needs)
+                needs.append(need)
             self._layout = CacheLayout(needs)
         return self._layout
 
