@@ -100,8 +100,11 @@ def retention(h, w_q, w_k, w_v, w_g, w_o, H, D, E, decay, eps, positions, rot):
     """Linear attention with a fixed decay per head, token by token: S <- decay S + k v^T, o = S^T q;
     each head's o over its root mean square, times silu of a gate, then the output matrix."""
     T = h.shape[0]
-    q = rotate((h @ w_q.T).view(T, H, D), positions, rot["dims"], rot["base"], rot.get("scaling"))
-    k = rotate((h @ w_k.T).view(T, H, D), positions, rot["dims"], rot["base"], rot.get("scaling")) * D ** -0.5
+    q, k = (h @ w_q.T).view(T, H, D), (h @ w_k.T).view(T, H, D)
+    if rot is not None:
+        q = rotate(q, positions, rot["dims"], rot["base"], rot.get("scaling"))
+        k = rotate(k, positions, rot["dims"], rot["base"], rot.get("scaling"))
+    k = k * D ** -0.5
     v = (h @ w_v.T).view(T, H, E)
     g = h @ w_g.T
     state = h.new_zeros(H, D, E)
@@ -141,7 +144,7 @@ def forward(config, weights, tokens, dtype=torch.float64, layers_out=None):
                                  m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["scale"], positions, m["rot"])
         elif layer["type"] == "retention":
             y = retention(x, w[p + "mix.q"], w[p + "mix.k"], w[p + "mix.v"], w[p + "mix.g"], w[p + "mix.o"],
-                          m["heads"], m["dim"], m["vdim"], m["decay"], eps, positions, m["rot"])
+                          m["heads"], m["dim"], m["vdim"], m["decay"], eps, positions, m.get("rot"))
         else:
             raise ValueError(layer["type"])
         x = rms_norm(alpha * x + w[p + "ls1"] * y, w[p + "norm1"], eps)
