@@ -70,8 +70,10 @@ class Retention(Mixer):
         cos, sin = self.position.tables(ctx)
         result = ctx.scratch("retention.o", (n, H * Ep), torch.float32)
         state = ctx.cache.states[run.cache_slot][self.STATE]
-        ops.retention(proj, 0, H * Dp, 2 * H * Dp, cos, sin, self.decay, state, ctx.q_start, ctx.state_slots, ctx.n_seqs,
-                      max(ctx.max_q_len, 1), result, self.dim ** -0.5)
+        for seq0, count, chunked in ((0, ctx.n_decode, False), (ctx.n_decode, ctx.n_seqs - ctx.n_decode, True)):
+            if count:       # one-token sequences walk token by token; prompt portions in chunks on the matrix unit
+                ops.retention(proj, 0, H * Dp, 2 * H * Dp, cos, sin, self.decay, state, ctx.q_start, ctx.state_slots, seq0,
+                              count, result, self.dim ** -0.5, chunked=chunked)
         act = ctx.scratch("retention.act", (n, H * Ep))
         ops.unit_gate(result, proj[:, 2 * H * Dp + H * Ep:], act, H, self.value_dim, Ep, self.eps)
         if ctx.defer_sums and self.o.deferrable(n):
