@@ -19,7 +19,7 @@ as the weights; `prefill_32k_prompts`: tokens a second over those prompts, which
 go through in portions of 2,048); and 1,024-token prompts with 512 generated tokens at batch 1, 8 and 64
 (`gen512_b*`, decoded tokens a second over the generated part).
 
-Other sizes of the architecture: --shape 14b|32b. --design kanavik measures the Kanavik
+Other sizes of the architecture: --shape 14b|32b. --design kanavik|dinutar measures that
 design's prefill and decode at a few layer sizes, each beside the Qwen2 decoder at equal
 width, heads, feed-forward and depth (one JSON line a size). --serve measures continuous
 batching under Poisson arrivals instead (prompts of 128..4,096 tokens, 256
@@ -89,7 +89,7 @@ def parse():
                    help="with --serve: the largest prompt portion in one step (larger: more prompt tokens a second and "
                         "a shorter time to the first token, longer steps for the requests that are decoding)")
     p.add_argument("--rate", type=float, default=16.0, help="mean arrivals a second (0: all at once)")
-    p.add_argument("--design", default="", choices=["", "kanavik"],
+    p.add_argument("--design", default="", choices=["", "kanavik", "dinutar"],
                    help="instead: prefill and decode throughput of another design at a few layer sizes (--design-sizes), "
                         "each beside the Qwen2 decoder at equal width, heads, feed-forward and depth; one JSON line a size")
     p.add_argument("--design-sizes", default="1b,3b,7b", help="which of the design's sizes to run, comma separated")
@@ -115,6 +115,35 @@ def kanavik_config(size, layers, context):
             "layers": [layer] * layers}
 
 
+# The Dinutar design at those widths: layers in the order retention, latent attention, retention, latent attention that
+# reads the cache of the one before; retention with half the heads, keys of the head size and values twice as wide (heads x
+# values = width); latent attention with the size's heads, 64 unrotated + 64 rotated query/key elements a head, values of
+# the head size, a latent of 192 (latent + rotated part: the 256 key elements the attention kernel takes).
+def dinutar_config(size, layers, context):
+    width, heads, _, dim, ff, _ = DESIGN_SIZES[size]
+    rot = {"base": 10000.0, "dims": 64, "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}
+    rheads = max(1, heads // 2)
+    decay = [1.0 - 2.0 ** (-5 - 3 * h / max(1, rheads - 1)) for h in range(rheads)]
+    mlp = {"kind": "dense", "ff": ff}
+
+    def latent(source):
+        m = {"heads": heads, "dim": dim - 64, "rot_dim": 64, "vdim": dim, "kv_rank": 192, "scale": dim ** -0.5, "rot": rot}
+        if source is not None:
+            m["kv_from"] = source
+        return {"type": "latent_attention", "mixer": m, "mlp": mlp}
+
+    out = []
+    for i in range(layers):
+        if i % 2 == 0:
+            out.append({"type": "retention", "mlp": mlp,
+                        "mixer": {"heads": rheads, "dim": dim, "vdim": width // rheads, "decay": decay,
+                                  "rot": {"base": 10000.0, "dims": dim}}})
+        else:
+            out.append(latent(i - 2 if i % 4 == 3 else None))
+    return {"architecture": "Dinutar", "vocab": DESIGN_VOCAB, "width": width, "norm": {"eps": 1e-6}, "postln_alpha": 1.0,
+            "embedding": {"scale": 1.0, "bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 7}}, "layers": out}
+
+
 def qwen2_config_like(size, layers, context):
     width, heads, kv_heads, dim, ff, _ = DESIGN_SIZES[size]
     return dict(QWEN25_7B, num_hidden_layers=layers, hidden_size=width, num_attention_heads=heads,
@@ -134,7 +163,8 @@ def design_run(args, torch):
                 "sizes": dict(zip(("width", "heads", "kv_heads", "head_dim", "ff", "window"), DESIGN_SIZES[size])),
                 "batch": args.batch, "context": args.context, "prefill_tokens": args.prefill_tokens,
                 "data": "synthetic: uniform-random token ids, random weights"}
-        models = [(args.design, kanavik_config(size, args.design_layers, args.context))]
+        make = {"kanavik": kanavik_config, "dinutar": dinutar_config}[args.design]
+        models = [(args.design, make(size, args.design_layers, args.context))]
         if not args.design_only:
             models.append(("qwen2", qwen2_config_like(size, args.design_layers, args.context)))
         for name, cfg in models:

@@ -55,7 +55,8 @@ _SIGNATURES = {
     "tw_embed_hashed": (I, [I, P, P, I, P, P, P, P, P, P, P, P, I, I, I, I, L, L, L, F, F, P, P, P]),
     "tw_latent_finish": (I, [I, P, L, I, I, I, P, P, P, P, L, P, P, P, I, I, I, I, I, I, I, F, P]),
     "tw_head_linear": (I, [I, P, L, I, P, P, L, I, I, I, I, I, P]),
-    "tw_retention": (I, [I, P, L, I, I, I, P, P, I, P, P, P, P, P, L, I, I, I, I, I, I, F, P]),
+    "tw_retention_workspace_floats": (L, [I, I, I, I, I]),
+    "tw_retention": (I, [I, P, L, I, I, I, P, P, I, P, P, P, P, P, L, I, I, I, I, I, I, F, P, L, P]),
     "tw_unit_gate": (I, [I, P, L, P, L, P, L, I, I, I, I, F, P]),
     "tw_sampling_uniform": (F, [c_uint64, c_uint64]),
     "tw_sample_workspace_bytes": (L, [I]),

@@ -832,13 +832,20 @@ def head_linear(x, x_stride, weight, out, out_stride):
 
 # ---- retention ------------------------------------------------------------------------------------------------
 
+def retention_workspace_floats(n_seqs, max_q_len, heads, key_dev, value_dev):
+    """float32 scratch the chunked retention kernel needs for portions of up to max_q_len tokens (0: none): long
+    portions are cut into segments for separate workgroups, which leave their partial states there."""
+    return int(library().tw_retention_workspace_floats(int(n_seqs), int(max_q_len), int(heads), int(key_dev), int(value_dev)))
+
+
 def retention(proj, q_col, k_col, v_col, cos, sin, decay, state, q_start, state_slots, seq0, n_seqs, out, k_scale,
-              chunked=True):
+              max_q_len=0, workspace=None):
     """S_t = decay_h S_(t-1) + k_t v_t^T, o_t = S_t^T q_t per head for sequences seq0 .. seq0 + n_seqs - 1, from and to
     state float32 [requests, H, Dp, Ep]. q, k (unrotated) and v are columns of proj (head h at col + h * Dp, or
     + h * Ep); they are rotated with cos/sin float32 [n, rot / 2] (None: no rotation) and k then multiplied by k_scale.
-    out float32 [n, H * Ep]. chunked: the kernel that walks a sequence's rows in chunks on the matrix unit (prompt
-    portions); else the one that walks them token by token (one-token steps)."""
+    out float32 [n, H * Ep]. max_q_len > 0: the kernel that walks a sequence's rows in chunks on the matrix unit, for
+    portions of up to that many tokens (with a workspace of `retention_workspace_floats` floats where that is not
+    zero); 0: the one that walks them token by token (one-token steps)."""
     n, width, ld = _rows(proj, "proj")
     _need(state.dim() == 4 and state.is_contiguous() and state.dtype == torch.float32, "state must be float32 [requests, H, Dp, Ep]")
     H, Dp, Ep = state.shape[1:]
@@ -854,10 +861,15 @@ def retention(proj, q_col, k_col, v_col, cos, sin, decay, state, q_start, state_
     _need(decay.numel() == H and decay.dtype == torch.float32, "one float32 decay per head")
     _need(seq0 >= 0 and q_start.numel() >= seq0 + n_seqs + 1 and state_slots.numel() >= seq0 + n_seqs, "sequence metadata is too short")
     _need(ldo % 4 == 0 and out.data_ptr() % 16 == 0, "out rows must be 16-byte aligned")
+    need = retention_workspace_floats(n_seqs, max_q_len, H, Dp, Ep) if max_q_len > 0 else 0
+    if need:
+        _need(workspace is not None and workspace.dtype == torch.float32 and workspace.is_contiguous() and workspace.numel() >= need,
+              "long portions need a float32 workspace of retention_workspace_floats floats")
     check(library().tw_retention(dtype_id(proj.dtype), _dev(proj), ld, int(q_col), int(k_col), int(v_col),
                                  _dev(cos) if rot else None, _dev(sin) if rot else None, rot, _dev(decay), _dev(state),
                                  _dev(q_start, torch.int32, "q_start"), _dev(state_slots, torch.int32, "state_slots"),
-                                 _dev(out), ldo, int(seq0), int(n_seqs), 1 if chunked else 0, H, Dp, Ep, float(k_scale), _stream()),
+                                 _dev(out), ldo, int(seq0), int(n_seqs), int(max_q_len), H, Dp, Ep, float(k_scale),
+                                 _dev(workspace) if need else None, workspace.numel() if need else 0, _stream()),
           "retention")
     return out
 

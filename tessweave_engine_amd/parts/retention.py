@@ -70,10 +70,14 @@ class Retention(Mixer):
         cos, sin = self.position.tables(ctx)
         result = ctx.scratch("retention.o", (n, H * Ep), torch.float32)
         state = ctx.cache.states[run.cache_slot][self.STATE]
-        for seq0, count, chunked in ((0, ctx.n_decode, False), (ctx.n_decode, ctx.n_seqs - ctx.n_decode, True)):
-            if count:       # one-token sequences walk token by token; prompt portions in chunks on the matrix unit
-                ops.retention(proj, 0, H * Dp, 2 * H * Dp, cos, sin, self.decay, state, ctx.q_start, ctx.state_slots, seq0,
-                              count, result, self.dim ** -0.5, chunked=chunked)
+        common = (proj, 0, H * Dp, 2 * H * Dp, cos, sin, self.decay, state, ctx.q_start, ctx.state_slots)
+        if ctx.n_decode:         # one-token sequences walk token by token
+            ops.retention(*common, 0, ctx.n_decode, result, self.dim ** -0.5)
+        portions = ctx.n_seqs - ctx.n_decode
+        if portions:             # prompt portions in chunks on the matrix unit, long ones cut into segments
+            floats = ops.retention_workspace_floats(portions, ctx.max_q_len, H, Dp, Ep)
+            ws = ctx.workspace.get("retention.segments", (floats,), torch.float32) if floats else None
+            ops.retention(*common, ctx.n_decode, portions, result, self.dim ** -0.5, max_q_len=ctx.max_q_len, workspace=ws)
         act = ctx.scratch("retention.act", (n, H * Ep))
         ops.unit_gate(result, proj[:, 2 * H * Dp + H * Ep:], act, H, self.value_dim, Ep, self.eps)
         if ctx.defer_sums and self.o.deferrable(n):

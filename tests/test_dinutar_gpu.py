@@ -159,6 +159,8 @@ def retention_case(H, D, E, rot_dims, decay, lengths, seed):
     (1, 128, 32, 0, [0.97], [[17, 130], [147]]),                            # no rotation, portions longer than any chunk
     (4, 32, 144, 32, [0.8, 0.9, 0.95, 0.995], [[200, 1, 1], [64, 64, 74]]),
     (1, 256, 48, 64, [0.999], [[33, 31, 70]]),                              # the longest keys: chunks of 32
+    (2, 64, 64, 64, [0.99, 0.9999], [[1500, 3, 300], [5, 700, 1098]]),      # long portions: several segments a sequence
+    (1, 128, 16, 32, [0.995], [[2304]]),
 ])
 def test_retention_over_portions(device, dtype, H, D, E, rot_dims, decay, cuts, chunked):
     """Sequences cut differently run side by side, step after step, from state slots that held other values; the
@@ -188,8 +190,11 @@ def test_retention_over_portions(device, dtype, H, D, E, rot_dims, decay, cuts, 
             sin = torch.empty_like(cos)
             ops.rope_table(pos, f, cos, sin)
         o = torch.empty(rows.shape[0], H * E, device=device)
+        longest = max(counts) if chunked else 0
+        floats = ops.retention_workspace_floats(len(live), longest, H, D, E) if chunked else 0
+        ws = torch.full((floats,), float("nan"), device=device) if floats else None
         ops.retention(rows, 0, H * D, 2 * H * D, cos, sin, dec, state, q_start, ints([slots[i] for i in live], device),
-                      0, len(live), o, D ** -0.5, chunked=chunked)
+                      0, len(live), o, D ** -0.5, max_q_len=longest, workspace=ws)
         act = torch.empty(rows.shape[0], H * E, dtype=dt, device=device)
         ops.unit_gate(o, rows[:, 2 * H * D + H * E:], act, H, E, E, 1e-5)
         row = 0
@@ -199,7 +204,7 @@ def test_retention_over_portions(device, dtype, H, D, E, rot_dims, decay, cuts, 
             row += n
     for i in range(len(cuts)):
         err = (got[i].double() - wants[i]).abs().max().item()
-        assert err < (4e-2 if dtype == "bfloat16" else 2e-4), (i, err)
+        assert err < (4e-2 if dtype == "bfloat16" else 5e-4), (i, err)      # (sums over up to 2,300 tokens at decays near one)
 
 
 def test_unit_gate_pads(device):
