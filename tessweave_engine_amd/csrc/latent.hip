@@ -21,6 +21,8 @@ struct LatentFinishArgs {
   const float* cos_t; const float* sin_t;    // [n][rot / 2]
   const float* norm_w;              // [L]
   void* q_out; long ld_q;           // [n][H][Lp + Rp]: this kernel fills columns Lp .. Lp + Rp of every head
+  void* q_full; long ld_full;       // or null. [n][H][hd]: head a = [its D unrotated elements | its rotated part | zeros],
+  int D, Dp, hd, full_from;         // for rows from full_from on (queries against keys expanded per head)
   void* keys; void* values;         // keys [pages][1][P][Lp + Rp], values [pages][1][Lp][P]; null: nothing is stored
   const int* slots;
   int H, L, Lp, Rp, rot, P;
@@ -52,6 +54,17 @@ __global__ __launch_bounds__(256) void latent_finish_kernel(LatentFinishArgs a) 
       v = tw_to_float(src[d]);
     }
     q[(size_t)head * K + a.Lp + d] = tw_from_float<T>(v);
+  }
+  if (a.q_full && n >= a.full_from) {
+    __syncthreads();                                                          // the rotated parts above, written by other threads
+    T* qf = (T*)a.q_full + (size_t)n * a.ld_full;
+    for (int i = threadIdx.x; i < a.H * a.hd; i += blockDim.x) {
+      const int head = i / a.hd, d = i % a.hd;
+      T v = tw_from_float<T>(0.f);
+      if (d < a.D) v = row[head * a.Dp + d];                                   // (the unrotated parts lie first in the row)
+      else if (d < a.D + a.rot) v = q[(size_t)head * K + a.Lp + d - a.D];
+      qf[i] = v;
+    }
   }
   if (!a.keys) return;
   const int slot = a.slots[n];
@@ -90,17 +103,19 @@ __global__ __launch_bounds__(256) void latent_finish_kernel(LatentFinishArgs a) 
 
 extern "C" int tw_latent_finish(int dtype, const void* proj, long ld, int q_col, int c_col, int kr_col,
                                 const float* cos_t, const float* sin_t, const float* norm_w, void* q_out, long ld_q,
+                                void* q_full, long ld_full, int D, int Dp, int hd, int full_from,
                                 void* keys, void* values, const int* slots, int n, int H, int L, int Lp, int Rp, int rot,
                                 int page_size, float eps, hipStream_t stream) {
   TW_REQUIRE(proj && cos_t && sin_t && q_out && n >= 0 && H > 0 && Rp > 0 && rot > 0 && rot % 2 == 0 && rot <= Rp);
+  if (q_full) TW_REQUIRE(D > 0 && Dp >= D && hd >= D + rot && ld_full >= (long)H * hd && full_from >= 0 && q_col >= H * Dp);
   TW_REQUIRE(q_col >= 0 && ld >= q_col + (long)H * Rp && ld_q >= (long)H * (Lp + Rp) && Lp >= 0);
   if (keys) {
     TW_REQUIRE(values && slots && norm_w && L > 0 && Lp >= L && page_size > 0 && eps > 0.f);
     TW_REQUIRE(c_col >= 0 && kr_col >= 0 && ld >= c_col + (long)L && ld >= kr_col + (long)rot);
   }
   if (n == 0) return 0;
-  LatentFinishArgs a{proj, ld, q_col, c_col, kr_col, cos_t, sin_t, norm_w, q_out, ld_q, keys, values, slots,
-                     H, L, Lp, Rp, rot, page_size, eps};
+  LatentFinishArgs a{proj, ld, q_col, c_col, kr_col, cos_t, sin_t, norm_w, q_out, ld_q, q_full, ld_full, D, Dp, hd, full_from,
+                     keys, values, slots, H, L, Lp, Rp, rot, page_size, eps};
   if (dtype == TW_DTYPE_BF16) latent_finish_kernel<bf16_t><<<n, 256, 0, stream>>>(a);
   else if (dtype == TW_DTYPE_F32) latent_finish_kernel<float><<<n, 256, 0, stream>>>(a);
   else return TW_ERR_BAD_ARGUMENT;
@@ -168,5 +183,97 @@ extern "C" int tw_head_linear(int dtype, const void* x, long ldx, int sx, const 
   else
     head_linear_kernel<float><<<grid, 256, 0, stream>>>((const float*)x, ldx, sx, (const float*)w, (float*)out, ldo, so, n,
                                                         heads, Ni, No, col_groups);
+  return TW_LAUNCH_RESULT();
+}
+
+// ---- prompt portions: keys and values expanded per head for this step ------------------------------------------------
+// Against many query rows it is cheaper to expand the cached latents once (k_a = W_uk,a c, v_a = W_uv,a c for every
+// cached token of the sequences that bring a portion) and to run ordinary attention with one key/value head per
+// query head than to carry the latent's size through every score. Two kernels around one matrix product:
+//
+//   latent_gather:        the key rows [c | kr] of sequences seq0 .. from their pages into rows of their own, sequence
+//                         after sequence, each starting at a multiple of the page size (row = page of its own * P + place),
+//                         and the block table of those pages
+//   (product)             up[row] = [W_uk ; W_uv] c[row]
+//   latent_expand_store:  keys [page][a][place][hd] = [up k-part of head a | kr | zeros], values [page][a][hd][place]
+//                         = [up v-part | zeros]: the layout the attention kernels read
+struct LatentGatherArgs {
+  const void* keys;                  // [pages][1][P][K]
+  const int* block_table; int table_stride;
+  const int* kv_len; const int* kv_page_start;      // kv_page_start[s]: pages of their own before sequence s (all sequences of the step)
+  void* rows;                        // [own pages * P][K]
+  int* own_table; int own_stride;    // [>= seq0 + n_seqs][own_stride]
+  int seq0, n_seqs, P, K;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void latent_gather_kernel(LatentGatherArgs a) {
+  const int base = a.kv_page_start[a.seq0];
+  const int pg = blockIdx.x;                                   // page of its own, counted from seq0's first
+  int lo = a.seq0, hi = a.seq0 + a.n_seqs - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (a.kv_page_start[mid] - base <= pg) lo = mid; else hi = mid - 1;
+  }
+  const int s = lo, b = pg - (a.kv_page_start[s] - base);
+  if (pg >= a.kv_page_start[a.seq0 + a.n_seqs] - base) return;
+  if (threadIdx.x == 0) a.own_table[(size_t)s * a.own_stride + b] = pg;
+  const int phys = a.block_table[(size_t)s * a.table_stride + b];
+  const int live = min(a.P, a.kv_len[s] - b * a.P);
+  const T* src = (const T*)a.keys + (size_t)(phys < 0 ? 0 : phys) * a.P * a.K;
+  T* dst = (T*)a.rows + (size_t)pg * a.P * a.K;
+  for (int i = threadIdx.x; i < a.P * a.K; i += blockDim.x)
+    dst[i] = (phys >= 0 && i / a.K < live) ? src[i] : tw_from_float<T>(0.f);
+}
+
+extern "C" int tw_latent_gather(int dtype, const void* keys, const int* block_table, int table_stride, const int* kv_len,
+                                const int* kv_page_start, void* rows, int* own_table, int own_stride, int seq0, int n_seqs,
+                                int own_pages, int page_size, int K, hipStream_t stream) {
+  TW_REQUIRE(keys && block_table && kv_len && kv_page_start && rows && own_table && seq0 >= 0 && n_seqs >= 0 && own_pages >= 0);
+  TW_REQUIRE(page_size > 0 && K > 0 && own_stride > 0);
+  if (n_seqs == 0 || own_pages == 0) return 0;
+  LatentGatherArgs a{keys, block_table, table_stride, kv_len, kv_page_start, rows, own_table, own_stride, seq0, n_seqs, page_size, K};
+  if (dtype == TW_DTYPE_BF16) latent_gather_kernel<bf16_t><<<own_pages, 256, 0, stream>>>(a);
+  else if (dtype == TW_DTYPE_F32) latent_gather_kernel<float><<<own_pages, 256, 0, stream>>>(a);
+  else return TW_ERR_BAD_ARGUMENT;
+  return TW_LAUNCH_RESULT();
+}
+
+// One workgroup a page: up [rows][H * D + H * E] (the heads' key parts, then their value parts), kr at rows[row][Lp ..].
+template <typename T>
+__global__ __launch_bounds__(256) void latent_expand_store_kernel(const T* __restrict__ up, long ld_up, const T* __restrict__ rows,
+                                                                  int K, int Lp, T* __restrict__ keys, T* __restrict__ values,
+                                                                  int H, int D, int R, int E, int hd, int P) {
+  const int pg = blockIdx.x;
+  T* kp = keys + (size_t)pg * H * P * hd;
+  T* vp = values + (size_t)pg * H * hd * P;
+  for (int i = threadIdx.x; i < H * P * hd; i += blockDim.x) {
+    const int d = i % hd, t = (i / hd) % P, a = i / (hd * P);
+    const size_t row = (size_t)pg * P + t;
+    T v = tw_from_float<T>(0.f);
+    if (d < D) v = up[row * ld_up + a * D + d];
+    else if (d < D + R) v = rows[row * K + Lp + d - D];
+    kp[i] = v;
+  }
+  for (int i = threadIdx.x; i < H * hd * P; i += blockDim.x) {
+    const int t = i % P, e = (i / P) % hd, a = i / (P * hd);
+    const size_t row = (size_t)pg * P + t;
+    vp[i] = e < E ? up[row * ld_up + (size_t)H * D + a * E + e] : tw_from_float<T>(0.f);
+  }
+}
+
+extern "C" int tw_latent_expand_store(int dtype, const void* up, long ld_up, const void* rows, int K, int Lp, void* keys,
+                                      void* values, int own_pages, int H, int D, int R, int E, int hd, int page_size,
+                                      hipStream_t stream) {
+  TW_REQUIRE(up && rows && keys && values && own_pages >= 0 && H > 0 && D > 0 && R >= 0 && E > 0 && page_size > 0);
+  TW_REQUIRE(hd >= D + R && hd >= E && ld_up >= (long)H * (D + E) && K >= Lp + R);
+  if (own_pages == 0) return 0;
+  if (dtype == TW_DTYPE_BF16)
+    latent_expand_store_kernel<bf16_t><<<own_pages, 256, 0, stream>>>((const bf16_t*)up, ld_up, (const bf16_t*)rows, K, Lp,
+                                                                      (bf16_t*)keys, (bf16_t*)values, H, D, R, E, hd, page_size);
+  else if (dtype == TW_DTYPE_F32)
+    latent_expand_store_kernel<float><<<own_pages, 256, 0, stream>>>((const float*)up, ld_up, (const float*)rows, K, Lp,
+                                                                     (float*)keys, (float*)values, H, D, R, E, hd, page_size);
+  else return TW_ERR_BAD_ARGUMENT;
   return TW_LAUNCH_RESULT();
 }

@@ -109,6 +109,7 @@ class Stepper:
         add("kv_len", max_seqs)
         add("state_slots", max_seqs)
         add("state_phase", max_seqs)
+        add("kv_page_start", max_seqs + 1)
         add("logit_rows", max_tokens)
         for g in range(n_groups):
             add(f"slots{g}", max_tokens)
@@ -286,6 +287,9 @@ class Stepper:
         put("state_phase", np.fromiter((e.seq.steps & 1 for e in ordered), dtype=np.int64, count=n_seqs))
         put("logit_rows", np.asarray(rows, dtype=np.int64))
         page = self.cache.page_size
+        kv_page_start = np.zeros(n_seqs + 1, dtype=np.int64)
+        np.cumsum((kv_len + page - 1) // page, out=kv_page_start[1:])
+        put("kv_page_start", kv_page_start)
         width = self.cache.table_width
         for g in range(len(self.cache.pools)):
             tables = self.cache.table_rows[g][slots_of]                       # [n_seqs, width]
@@ -308,6 +312,8 @@ class Stepper:
         ctx.kv_len = self._dev("kv_len", n_seqs)
         ctx.state_slots = self._dev("state_slots", n_seqs)
         ctx.state_phase = self._dev("state_phase", n_seqs)
+        ctx.kv_page_start = self._dev("kv_page_start", n_seqs + 1)
+        ctx.h_kv_page_start = kv_page_start.tolist()
         ctx.logit_rows = self._dev("logit_rows", n_logits)
         ctx.groups = [GroupStep(self._dev(f"table{g}", n_seqs * width).view(n_seqs, width),
                                 self._dev(f"slots{g}", n_tokens)) for g in range(len(self.cache.pools))]

@@ -782,11 +782,13 @@ def embed_hashed(ids, table, pairs, norm_weight, q_start, kv_len, state_slots, p
 # ---- attention over a cached latent: finishing a token's projections, one small matrix per head -----------------------
 
 def latent_finish(proj, q_col, c_col, kr_col, cos, sin, norm_weight, q_out, heads, latent, latent_dev, rot_dev, eps,
-                  keys=None, values=None, slots=None):
+                  keys=None, values=None, slots=None, q_full=None, dim=0, dim_dev=0, full_from=0):
     """Rotates the heads' rotated query parts proj[n, q_col + a * rot_dev ...] into q_out[n, a, latent_dev:], and,
     with keys/values, stores the token's key row [unit(proj[n, c_col : c_col + latent]) * norm_weight | zeros |
     rotated proj[n, kr_col ...] | zeros] and its value (the normed latent) into page slot slots[n] (-1: not stored).
-    keys [pages, 1, page, latent_dev + rot_dev]; values [pages, 1, latent_dev, page]; q_out [n, heads * (latent_dev + rot_dev)]."""
+    keys [pages, 1, page, latent_dev + rot_dev]; values [pages, 1, latent_dev, page]; q_out [n, heads * (latent_dev + rot_dev)].
+    q_full [n, heads * hd]: rows from full_from on also get whole query heads [the head's dim unrotated elements (which lie
+    first in proj, dim_dev apart) | its rotated part | zeros], for attention against keys expanded per head."""
     n, width, ld = _rows(proj, "proj")
     rot = 2 * cos.shape[1]
     _need(tuple(cos.shape) == (n, rot // 2) and tuple(sin.shape) == (n, rot // 2) and cos.is_contiguous() and sin.is_contiguous()
@@ -804,11 +806,51 @@ def latent_finish(proj, q_col, c_col, kr_col, cos, sin, norm_weight, q_out, head
         _need(slots.numel() == n and norm_weight.numel() == latent and norm_weight.dtype == torch.float32 and latent <= latent_dev,
               "one slot per token and a float32 norm weight per latent element are needed")
         _need(c_col + latent <= width and kr_col + rot <= width, "the latent or the shared key part exceed the projection's row")
+    ld_full = hd = 0
+    if q_full is not None:
+        nf, wf, ld_full = _rows(q_full, "q_full")
+        hd = wf // heads
+        _need(nf == n and wf == heads * hd and q_full.dtype == proj.dtype and hd >= dim + rot and dim_dev >= dim > 0
+              and q_col >= heads * dim_dev, "q_full must be [n, heads * hd] with hd >= dim + rot")
     check(library().tw_latent_finish(dtype_id(proj.dtype), _dev(proj), ld, int(q_col), int(c_col), int(kr_col), _dev(cos), _dev(sin),
                                      _dev(norm_weight) if keys is not None else None, _dev(q_out), ldq,
-                                     _dev(keys) if keys is not None else None, _dev(values) if keys is not None else None,
+                                     _dev(q_full) if q_full is not None else None, ld_full, int(dim), int(dim_dev), int(hd),
+                                     int(full_from), _dev(keys) if keys is not None else None, _dev(values) if keys is not None else None,
                                      _dev(slots, torch.int32, "slots") if keys is not None else None, n, heads, int(latent),
                                      int(latent_dev), int(rot_dev), rot, page, float(eps), _stream()), "latent_finish")
+
+
+def latent_gather(keys, block_table, kv_len, kv_page_start, seq0, n_seqs, own_pages, rows, own_table):
+    """The cached key rows of sequences seq0 .. seq0 + n_seqs - 1 from their pages into pages of their own, sequence after
+    sequence (own page kv_page_start[s] - kv_page_start[seq0] + b holds block b of sequence s; places past a sequence's
+    end are zeros), and those pages' numbers into own_table[s, b]. keys [pages, 1, page, K]; rows [own_pages * page, K]."""
+    page, K = keys.shape[2], keys.shape[3]
+    _need(keys.dim() == 4 and keys.shape[1] == 1 and keys.is_contiguous(), "keys must be contiguous [pages, 1, page, K]")
+    _need(rows.is_contiguous() and tuple(rows.shape) == (own_pages * page, K) and rows.dtype == keys.dtype, "rows must be [own_pages * page, K]")
+    _need(own_table.dtype == torch.int32 and own_table.dim() == 2 and own_table.stride(1) == 1 and own_table.shape[0] >= seq0 + n_seqs,
+          "own_table must be int32 [sequences, blocks]")
+    _need(block_table.dim() == 2 and block_table.stride(1) == 1 and block_table.shape[0] >= seq0 + n_seqs
+          and own_table.shape[1] >= block_table.shape[1], "block_table must be 2-D and own_table as wide")
+    _need(kv_len.numel() >= seq0 + n_seqs and kv_page_start.numel() >= seq0 + n_seqs + 1, "sequence metadata is too short")
+    check(library().tw_latent_gather(dtype_id(keys.dtype), _dev(keys), _dev(block_table, torch.int32, "block_table"),
+                                     block_table.stride(0), _dev(kv_len, torch.int32, "kv_len"),
+                                     _dev(kv_page_start, torch.int32, "kv_page_start"), _dev(rows), _dev(own_table),
+                                     own_table.stride(0), int(seq0), int(n_seqs), int(own_pages), page, K, _stream()), "latent_gather")
+
+
+def latent_expand_store(up, rows, latent_dev, keys, values, heads, dim, rot, value_dim):
+    """keys[page, a, place] = [up[row, a * dim : (a + 1) * dim] | rows[row, latent_dev : latent_dev + rot] | zeros] and
+    values[page, a, :, place] = [up[row, heads * dim + a * value_dim ...] | zeros] for row = page * page_size + place.
+    keys [own_pages, heads, page, hd]; values [own_pages, heads, hd, page]."""
+    n, wu, ld_up = _rows(up, "up")
+    own_pages, H, page, hd = keys.shape
+    _need(H == heads and keys.is_contiguous() and values.is_contiguous() and tuple(values.shape) == (own_pages, H, hd, page)
+          and keys.dtype == up.dtype == rows.dtype == values.dtype, "keys [own_pages, heads, page, hd], values [own_pages, heads, hd, page]")
+    _need(n == own_pages * page and wu == heads * (dim + value_dim) and rows.is_contiguous() and rows.shape[0] == n
+          and rows.shape[1] >= latent_dev + rot and hd >= max(dim + rot, value_dim), "latent_expand_store shapes do not agree")
+    check(library().tw_latent_expand_store(dtype_id(up.dtype), _dev(up), ld_up, _dev(rows), rows.shape[1], int(latent_dev), _dev(keys),
+                                           _dev(values), own_pages, heads, int(dim), int(rot), int(value_dim), hd, page, _stream()),
+          "latent_expand_store")
 
 
 def head_linear(x, x_stride, weight, out, out_stride):

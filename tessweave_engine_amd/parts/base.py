@@ -218,6 +218,8 @@ class StepContext:
         self.state_slots = None      # int32 [n_seqs]
         self.state_phase = None      # int32 [n_seqs]: which of two copies of a double-buffered state is current (the
                                      # step reads that copy and writes the other; it alternates with every step of a request)
+        self.kv_page_start = None    # int32 [n_seqs + 1]: pages that the sequences before s would fill if every sequence's keys
+                                     # (this step's included) lay in pages of its own, one sequence after the other
         self.logit_rows = None       # int32 [n_logits]
         self.n_logits = 0
         self.groups = []             # GroupStep per cache group
@@ -225,6 +227,7 @@ class StepContext:
         self.h_q_start = []
         self.h_kv_len = []
         self.h_state_slots = []
+        self.h_kv_page_start = []
         self.max_q_len = 0           # over the sequences after the first n_decode
         self.max_kv_len = 0
         self.kv_capacity = 0         # most keys a sequence can ever hold (block-table width * page size)

@@ -5,10 +5,13 @@ head a's key is [W_uk,a c | kr], its value W_uv,a c, its query [D unrotated | R 
 
     score_a(i, j) = scale * (q_plain,a(i) . W_uk,a c_j + q_turned,a(i) . kr_j),   causal softmax,   out = W_o [.. W_uv,a sum_j p c_j ..]
 
-Only c and kr are cached. The products with W_uk and W_uv are moved to the query side and the output side (one
-small matrix per head each, `ops.head_linear`), so that the attention itself runs over one key/value head whose
-key row is [c | kr] and whose value is c, for all query heads at once; the engine's paged cache holds it like any
-other group (one key/value head, values of another size than keys). A layer may read the cache slot of another
+Only c and kr are cached; the engine's paged cache holds them like any other group (one key/value head whose key row
+is [c | kr] and whose value is c). One-token sequences run the attention over that one head directly, for all query
+heads at once: the products with W_uk and W_uv are moved to the query side and the output side (one small matrix per
+head each, `ops.head_linear`), so a step reads every cached token once, at the latent's size. Prompt portions, with
+many query rows against the same keys, go the other way round: the cached latents of their sequences are expanded
+once a step (one product with [W_uk; W_uv] over the gathered key rows) into keys and values per head in scratch pages
+of their own, and the engine's ordinary prompt attention runs on those. A layer may read the cache slot of another
 layer (`LayerRun(writes_cache=False)`): it then has no down-projection of its own (`own_latent=False`) and uses that
 layer's c and kr with its own queries and its own W_uk, W_uv.
 """
@@ -40,13 +43,15 @@ class LatentAttention(Mixer):
         if position.rotary_dim <= 0 or position.rotary_dim > self.rot_dim or position.pairing != "half":
             raise ValueError("the rotated part needs a rotary encoding of at most rot_dim elements with the 'half' pairing")
         # sizes on the device: tails of zeros, which add nothing to a product
-        self.dim_dev, self.value_dev = _round_up(dim, 8), _round_up(value_dim, 8)
+        self.dim_dev = _round_up(dim, 8)
         self.latent_dev, self.rot_dev = _round_up(latent, 16), _round_up(rot_dim, 16)
         self.key_dev = self.latent_dev + self.rot_dev
-        if self.heads > 32 or self.key_dev > 256:
-            raise ValueError("the attention kernel takes up to 32 heads and latent + rotated sizes up to 256")
+        # the size of an expanded head (prompt portions): keys [unrotated | rotated] and values side by side in one size
+        self.value_dev = self.head_dev = _round_up(max(self.dim + self.rot_dim, self.value_dim), 16)
+        if self.heads > 32 or self.key_dev > 256 or self.head_dev > 256:
+            raise ValueError("the attention kernels take up to 32 heads, latent + rotated sizes up to 256 and heads up to 256")
         self.scale, self.eps, self.position, self.own_latent = float(scale), float(eps), position, bool(own_latent)
-        self.proj = self.absorb = self.expand = self.latent_norm = None
+        self.proj = self.up = self.absorb = self.expand = self.latent_norm = None
         self.o = Linear([prefix + self.names[5]], heads * value_dim, [hidden], pad_in=(self.value_dim, self.value_dev),
                         suffixes=("", ".bias"))
 
@@ -54,6 +59,8 @@ class LatentAttention(Mixer):
         return self.prefix + self.names[i]
 
     def parts(self):
+        # (`up`, the matrix of the prompt path, is a second arrangement of W_uk and W_uv, which `weight_tensors` already
+        # names: a step reads one arrangement or the other, so it is not listed again)
         return [p for p in (self.proj, self.o, self.position) if p is not None]
 
     def tensor_specs(self):
@@ -89,6 +96,14 @@ class LatentAttention(Mixer):
         uv = tensors.pop(self._name(4)).view(H, E, L)
         self.expand = uv.new_zeros(H, Ep, Lp)
         self.expand[:, :E, :L] = uv
+        # prompt portions: [W_uk; W_uv] over the latent as one matrix (the heads' key parts, then their value parts)
+        both = uk.new_zeros(H * (D + E), Lp)
+        both[:H * D, :L] = uk.reshape(H * D, L)
+        both[H * D:, :L] = uv.reshape(H * E, L)
+        name = self.prefix + "expand"
+        self.up = Linear([name], Lp, [H * (D + E)])
+        self.up.bind({name + ".weight": both}, dtype, device)
+        del both
         self.o.bind(tensors, dtype, device)
         self.position.bind(tensors, dtype, device)
 
@@ -101,42 +116,53 @@ class LatentAttention(Mixer):
     def forward(self, ctx, run, h, x, accumulate=True):
         if run.writes_cache != self.own_latent:
             raise RuntimeError("a layer with a latent of its own writes its cache slot; one without reads another layer's")
-        n, H = ctx.n_tokens, self.heads
-        Lp, Rp, K = self.latent_dev, self.rot_dev, self.key_dev
+        n, H, nd = ctx.n_tokens, self.heads, ctx.n_decode
+        Lp, Rp, K, hd = self.latent_dev, self.rot_dev, self.key_dev, self.head_dev
+        portions = ctx.n_seqs - nd
         proj = ctx.scratch("latent.proj", (n, self.proj_width))
         self.proj.forward(ctx, h, proj)
         cos, sin = self.position.tables(ctx)
         keys, values, g = ctx.cache.keys_values(run.cache_slot)
-        values = values.view(values.shape[0], 1, Lp, ctx.cache.page_size)
+        page = ctx.cache.page_size
+        values = values.view(values.shape[0], 1, Lp, page)
         group = ctx.groups[g]
         q = ctx.scratch("latent.q", (n, H * K))
+        q_full = ctx.scratch("latent.q_full", (n, H * hd)) if portions else None
         store = dict(keys=keys, values=values, slots=group.slot_mapping) if self.own_latent else {}
         ops.latent_finish(proj, self.q_col, self.c_col, self.kr_col, cos, sin, self.latent_norm, q, H, self.latent, Lp, Rp,
-                          self.eps, **store)
-        ops.head_linear(proj, self.dim_dev, self.absorb, q, K)
-        mixed = ctx.scratch("latent.mixed", (n, H * Lp))
-        if ctx.n_decode:
+                          self.eps, q_full=q_full, dim=self.dim, dim_dev=self.dim_dev, full_from=nd, **store)
+        out = ctx.scratch("latent.out", (n, H * hd))
+        if nd:
+            # one-token sequences: all heads over the one cached head, W_uk on the query side, W_uv on the output side
+            ops.head_linear(proj[:nd], self.dim_dev, self.absorb, q[:nd], K)
+            mixed = ctx.scratch("latent.mixed", (n, H * Lp))[:nd]
             longest = ctx.kv_bound if ctx.capturing else ctx.max_kv_len
-            splits = ops.attn_mixed_splits(ctx.n_decode, longest)
+            splits = ops.attn_mixed_splits(nd, longest)
             ws = None
             if splits > 1:
                 # sized for the most splits any length class can ask for, so that it never grows under a capture
-                floats = ops.attn_mixed_workspace_floats(ctx.n_decode, 1, H, Lp,
-                                                         max(splits, ops.attn_mixed_splits(ctx.n_decode, ctx.kv_capacity)))
+                floats = ops.attn_mixed_workspace_floats(nd, 1, H, Lp, max(splits, ops.attn_mixed_splits(nd, ctx.kv_capacity)))
                 ws = ctx.workspace.get("attn.mixed.split", (floats,), torch.float32)
-            ops.attn_mixed(q, keys, values, group.block_table, ctx.q_start, ctx.kv_len, 0, ctx.n_decode, 1, mixed, H, 1,
+            ops.attn_mixed(q[:nd], keys, values, group.block_table, ctx.q_start, ctx.kv_len, 0, nd, 1, mixed, H, 1,
                            self.scale, splits=splits, workspace=ws)
-        if ctx.n_seqs > ctx.n_decode:
-            n_seqs = ctx.n_seqs - ctx.n_decode
-            splits = ops.attn_mixed_prefill_splits(ctx.n_tokens - ctx.n_decode, n_seqs, ctx.max_kv_len)
+            ops.head_linear(mixed, Lp, self.expand, out[:nd], hd)
+        if portions:
+            # prompt portions: their sequences' cached latents expanded per head into pages of this step's own
+            own_pages = ctx.h_kv_page_start[ctx.n_seqs] - ctx.h_kv_page_start[nd]
+            rows = ctx.workspace.get("latent.rows", (own_pages * page, K), ctx.dtype)
+            own_table = ctx.workspace.get("latent.table", (ctx.n_seqs, group.block_table.shape[1]), torch.int32)
+            ops.latent_gather(keys, group.block_table, ctx.kv_len, ctx.kv_page_start, nd, portions, own_pages, rows, own_table)
+            up = ctx.workspace.get("latent.up", (own_pages * page, H * (self.dim + self.value_dim)), ctx.dtype)
+            self.up.forward(ctx, rows[:, :Lp], up)
+            own_keys = ctx.workspace.get("latent.keys", (own_pages, H, page, hd), ctx.dtype)
+            own_values = ctx.workspace.get("latent.values", (own_pages, H, hd, page), ctx.dtype)
+            ops.latent_expand_store(up, rows, Lp, own_keys, own_values, H, self.dim, self.rot_dim, self.value_dim)
+            split = ops.attn_prefill_split(portions, H, H, ctx.max_q_len, ctx.max_kv_len)
             ws = None
-            if splits > 1:
-                floats = ops.attn_mixed_workspace_floats(n_seqs, ctx.max_q_len, H, Lp, splits)
-                ws = ctx.workspace.get("attn.mixed.split.rows", (floats,), torch.float32)
-            ops.attn_mixed(q, keys, values, group.block_table, ctx.q_start, ctx.kv_len, ctx.n_decode, n_seqs, ctx.max_q_len,
-                           mixed, H, 1, self.scale, splits=splits, workspace=ws)
-        out = ctx.scratch("latent.out", (n, H * self.value_dev))
-        ops.head_linear(mixed, Lp, self.expand, out, self.value_dev)
+            if split[0] > 1:
+                ws = ctx.workspace.get("attn.prefill_split", (ops.attn_prefill_workspace_floats(n, H, hd, split[0]),), torch.float32)
+            ops.attn_prefill(q_full, own_keys, own_values, own_table, ctx.q_start, ctx.kv_len, nd,
+                             portions, ctx.max_q_len, out, H, H, hd, self.scale, split=split, workspace=ws)
         if ctx.defer_sums and self.o.deferrable(n):
             return self.o.forward_partials(ctx, out, "o")          # whoever norms next adds them up
         self.o.forward(ctx, out, x, residual=x if accumulate else None)
