@@ -277,3 +277,230 @@ extern "C" int tw_latent_expand_store(int dtype, const void* up, long ld_up, con
   else return TW_ERR_BAD_ARGUMENT;
   return TW_LAUNCH_RESULT();
 }
+
+// ---- one-token sequences: all heads of a sequence against the one cached head ------------------------------------------
+// The query heads are the 16 columns of the matrix unit's tile (a launch has one workgroup row per 16 heads): per 16
+// keys a wave forms S^T = K Q^T (keys down, heads across), so every head's probabilities leave the product in the
+// layout the next one, O^T += V^T P^T, wants as its operand, and a key row is read once for 16 heads. Values are the
+// first Lp elements of the key rows, kept a second time transposed inside a page ([Lp][P]) so that four consecutive
+// keys of one element are one 8-byte load. A sequence's keys are cut into `splits` ranges for separate workgroups,
+// whose waves take the range's tiles in turn; waves are combined through LDS, ranges by a second kernel in index order.
+//
+//   part [seq][head tile][split][16][Lp + 2]: output sums relative to the range's maximum, that maximum, the sum
+struct LatentDecodeArgs {
+  const void* q; long ldq;            // head a of sequence s at q + row(s) * ldq + a * K
+  const void* keys; const void* values;
+  const int* block_table; int table_stride;
+  const int* q_start; const int* kv_len;
+  void* out; long ldo;                // head a at out + row(s) * ldo + a * Lp
+  float* part;
+  float scale;
+  int H, K, Lp, P, splits;
+};
+
+template <typename T> __device__ __forceinline__ float lt_exp(float v);
+template <> __device__ __forceinline__ float lt_exp<float>(float v) { return expf(v); }
+template <> __device__ __forceinline__ float lt_exp<bf16_t>(float v) { return __expf(v); }
+
+template <typename T> struct LtQuad;
+template <> struct LtQuad<float> { typedef f32x4 Type; };
+template <> struct LtQuad<bf16_t> { typedef bf16x4 Type; };
+
+template <typename T>
+__global__ __launch_bounds__(256) void latent_decode_kernel(LatentDecodeArgs a) {
+  typedef typename Elem<T>::Frag Frag;
+  typedef typename LtQuad<T>::Type Quad;
+  constexpr int EPF = Elem<T>::kPerFrag;
+  constexpr int STEP = 4 * EPF;                 // key elements one product consumes
+  constexpr int KC_MAX = 256 / STEP;
+  constexpr int LT_MAX = 15;                    // Lp <= 240
+  extern __shared__ float ld_lds[];
+  const int s = blockIdx.x, split = blockIdx.y, ht = blockIdx.z;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int K = a.K, Lp = a.Lp, P = a.P;
+  const int KC = (K + STEP - 1) / STEP, LT = Lp / 16;
+  const int len = a.kv_len[s];
+  const int row = a.q_start[s];
+  const int head = ht * 16 + r;
+  const int* table = a.block_table + (size_t)s * a.table_stride;
+  const T* keys = (const T*)a.keys;
+  const T* values = (const T*)a.values;
+  // this lane's query fragments: head r, elements kc * STEP + g * EPF ..
+  Frag qf[KC_MAX];
+#pragma unroll
+  for (int kc = 0; kc < KC_MAX; ++kc) {
+    const int col = kc * STEP + g * EPF;
+    qf[kc] = (kc < KC && col < K && head < a.H) ? tw_load_frag((const T*)a.q + (size_t)row * a.ldq + (size_t)head * K + col)
+                                                 : Elem<T>::zero();
+  }
+  f32x4 O[LT_MAX];
+#pragma unroll
+  for (int lt = 0; lt < LT_MAX; ++lt) O[lt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, sum = 0.f;
+  const int tiles = (len + 15) / 16;
+  const int per = (tiles + a.splits - 1) / a.splits;
+  const int t_begin = split * per, t_end = min(tiles, t_begin + per);
+  for (int t = t_begin + wave; t < t_end; t += 4) {
+    const bool edge = t * 16 + 16 > len;
+    // S^T for 16 keys: this lane loads key t * 16 + r (a key past the end stands in for by the last one; masked below)
+    const int pk = min(t * 16 + r, len - 1);
+    const T* krow = keys + ((size_t)table[pk / P] * P + pk % P) * K;
+    f32x4 S = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int kc = 0; kc < KC_MAX; ++kc) {
+      if (kc < KC) {
+        const int col = kc * STEP + g * EPF;
+        const Frag kf = col < K ? tw_load_frag(krow + col) : Elem<T>::zero();
+        tw_mma16(S, kf, qf[kc]);                  // S[j]: key t * 16 + 4 g + j against head r
+      }
+    }
+    // values of keys t * 16 + 4 g .. + 3 (one page: pages hold a multiple of 4 keys)
+    const int pv = min(t * 16 + 4 * g, (len - 1) / 4 * 4);
+    const T* vbase = values + (size_t)table[pv / P] * Lp * P + pv % P;
+    Quad vq[LT_MAX];
+#pragma unroll
+    for (int lt = 0; lt < LT_MAX; ++lt)
+      if (lt < LT) vq[lt] = *reinterpret_cast<const Quad*>(vbase + (size_t)(lt * 16 + r) * P);
+    float top = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      S[j] = (edge && t * 16 + 4 * g + j >= len) ? -INFINITY : S[j] * a.scale;
+      top = fmaxf(top, S[j]);
+    }
+    top = tw_rows_max(top);                      // over the 16 keys, for head r
+    const float m_new = fmaxf(m, top);
+    const float alpha = m == -INFINITY ? 0.f : lt_exp<T>(m - m_new);
+    f32x4 Pr;
+    float part = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      Pr[j] = S[j] == -INFINITY ? 0.f : lt_exp<T>(S[j] - m_new);
+      part += Pr[j];
+    }
+    sum = sum * alpha + tw_rows_sum(part);
+    m = m_new;
+#pragma unroll
+    for (int lt = 0; lt < LT_MAX; ++lt) {
+      if (lt < LT) {
+        Quad v = vq[lt];
+        if (edge) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            if (t * 16 + 4 * g + j >= len) v[j] = tw_from_float<T>(0.f);     // whatever lies there must not reach a sum
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) O[lt][j] *= alpha;
+        tw_mma16_k4(O[lt], v, Pr);               // O[lt][j]: element lt * 16 + 4 g + j of head r
+      }
+    }
+  }
+  // ---- the four waves' results through LDS: [wave][16 heads][Lp + 4] sums, then [wave][16] maxima and sums
+  const int OS = Lp + 4;
+  float* Ow = ld_lds;
+  float* mw = Ow + (size_t)4 * 16 * OS;
+  float* sw = mw + 64;
+#pragma unroll
+  for (int lt = 0; lt < LT_MAX; ++lt)
+    if (lt < LT) *reinterpret_cast<f32x4*>(Ow + ((size_t)wave * 16 + r) * OS + lt * 16 + 4 * g) = O[lt];
+  if (g == 0) {
+    mw[wave * 16 + r] = m;
+    sw[wave * 16 + r] = sum;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < 16 * Lp; i += 256) {
+    const int hh = i / Lp, l = i - hh * Lp;
+    if (ht * 16 + hh >= a.H) continue;
+    float top = fmaxf(fmaxf(mw[hh], mw[16 + hh]), fmaxf(mw[32 + hh], mw[48 + hh]));
+    float o = 0.f, total = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float f = mw[w * 16 + hh] == -INFINITY ? 0.f : lt_exp<T>(mw[w * 16 + hh] - top);
+      o += f * Ow[((size_t)w * 16 + hh) * OS + l];
+      total += f * sw[w * 16 + hh];
+    }
+    if (a.splits == 1) {
+      ((T*)a.out)[(size_t)row * a.ldo + (size_t)(ht * 16 + hh) * Lp + l] = tw_from_float<T>(o / total);
+    } else {
+      float* dst = a.part + ((((size_t)s * gridDim.z + ht) * a.splits + split) * 16 + hh) * (Lp + 2);
+      dst[l] = o;
+      if (l == 0) {
+        dst[Lp] = top;
+        dst[Lp + 1] = total;
+      }
+    }
+  }
+}
+
+// One workgroup a (sequence, head): the ranges' maxima and sums first (one thread a range), then a thread an element.
+template <typename T>
+__global__ __launch_bounds__(256) void latent_decode_merge_kernel(LatentDecodeArgs a) {
+  __shared__ float weight[64];
+  __shared__ float total_s;
+  const int s = blockIdx.x, head = blockIdx.y;
+  const int ht = head >> 4, hh = head & 15;
+  const int Lp = a.Lp;
+  const int row = a.q_start[s];
+  const int head_tiles = (a.H + 15) / 16;
+  const float* base = a.part + ((((size_t)s * head_tiles + ht) * a.splits) * 16 + hh) * (Lp + 2);
+  const size_t stride = (size_t)16 * (Lp + 2);                  // from one range to the next
+  if (threadIdx.x < 64) {
+    const int sp = threadIdx.x;
+    const float m = sp < a.splits ? base[sp * stride + Lp] : -INFINITY;
+    const float top = tw_wave_max(m);
+    const float f = m == -INFINITY ? 0.f : lt_exp<T>(m - top);
+    weight[sp] = f;
+    const float total = tw_wave_sum(sp < a.splits ? f * base[sp * stride + Lp + 1] : 0.f);
+    if (sp == 0) total_s = total;
+  }
+  __syncthreads();
+  const float inv = 1.f / total_s;
+  for (int l = threadIdx.x; l < Lp; l += 256) {
+    float o = 0.f;
+    for (int sp = 0; sp < a.splits; ++sp) o += weight[sp] * base[sp * stride + l];
+    ((T*)a.out)[(size_t)row * a.ldo + (size_t)head * Lp + l] = tw_from_float<T>(o * inv);
+  }
+}
+
+// Key ranges a sequence: enough workgroups for the chip, each range at least 8 tiles of 16 keys.
+extern "C" int tw_latent_decode_splits(int n_seqs, int heads, int max_kv_len) {
+  if (n_seqs <= 0) return 1;
+  const int tiles = tw_div_up(max_kv_len, 16);
+  int want = 512 / (n_seqs * tw_div_up(heads, 16));
+  if (want > tiles / 8) want = tiles / 8;
+  if (want > 64) want = 64;
+  return want < 1 ? 1 : want;
+}
+
+extern "C" long tw_latent_decode_workspace_floats(int n_seqs, int heads, int Lp, int splits) {
+  return splits > 1 ? (long)n_seqs * tw_div_up(heads, 16) * splits * 16 * (Lp + 2) : 0;
+}
+
+extern "C" int tw_latent_decode(int dtype, const void* q, long ldq, const void* keys, const void* values,
+                                const int* block_table, int table_stride, const int* q_start, const int* kv_len,
+                                int n_seqs, void* out, long ldo, float* workspace, long workspace_floats, int heads,
+                                int K, int Lp, int page_size, float scale, int splits, hipStream_t stream) {
+  TW_REQUIRE(q && keys && values && block_table && q_start && kv_len && out && n_seqs >= 0 && splits >= 1 && splits <= 64);
+  TW_REQUIRE(heads >= 1 && K % 16 == 0 && K <= 256 && Lp % 16 == 0 && Lp >= 16 && Lp <= 240 && Lp <= K);
+  TW_REQUIRE(page_size > 0 && page_size % 4 == 0);
+  TW_REQUIRE(ldq >= (long)heads * K && ldo >= (long)heads * Lp);
+  const int esize = dtype == TW_DTYPE_BF16 ? 2 : 4;
+  TW_REQUIRE((uintptr_t)q % 16 == 0 && (uintptr_t)keys % 16 == 0 && (uintptr_t)values % 16 == 0 && (ldq * esize) % 16 == 0);
+  if (splits > 1) TW_REQUIRE(workspace && workspace_floats >= tw_latent_decode_workspace_floats(n_seqs, heads, Lp, splits));
+  if (n_seqs == 0) return 0;
+  LatentDecodeArgs a{q, ldq, keys, values, block_table, table_stride, q_start, kv_len, out, ldo, workspace, scale,
+                     heads, K, Lp, page_size, splits};
+  const int head_tiles = tw_div_up(heads, 16);
+  const dim3 grid(n_seqs, splits, head_tiles);
+  const size_t lds = ((size_t)4 * 16 * (Lp + 4) + 128) * sizeof(float);
+  if (dtype == TW_DTYPE_BF16) {
+    latent_decode_kernel<bf16_t><<<grid, 256, lds, stream>>>(a);
+    if (splits > 1) latent_decode_merge_kernel<bf16_t><<<dim3(n_seqs, heads), 256, 0, stream>>>(a);
+  } else if (dtype == TW_DTYPE_F32) {
+    latent_decode_kernel<float><<<grid, 256, lds, stream>>>(a);
+    if (splits > 1) latent_decode_merge_kernel<float><<<dim3(n_seqs, heads), 256, 0, stream>>>(a);
+  } else {
+    return TW_ERR_BAD_ARGUMENT;
+  }
+  return TW_LAUNCH_RESULT();
+}

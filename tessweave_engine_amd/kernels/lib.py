@@ -54,6 +54,9 @@ _SIGNATURES = {
     "tw_relu_squared": (I, [I, P, L, I, I, P]),
     "tw_embed_hashed": (I, [I, P, P, I, P, P, P, P, P, P, P, P, I, I, I, I, L, L, L, F, F, P, P, P]),
     "tw_latent_finish": (I, [I, P, L, I, I, I, P, P, P, P, L, P, L, I, I, I, I, P, P, P, I, I, I, I, I, I, I, F, P]),
+    "tw_latent_decode_splits": (I, [I, I, I]),
+    "tw_latent_decode_workspace_floats": (L, [I, I, I, I]),
+    "tw_latent_decode": (I, [I, P, L, P, P, P, I, P, P, I, P, L, P, L, I, I, I, I, F, I, P]),
     "tw_latent_gather": (I, [I, P, P, I, P, P, P, P, I, I, I, I, I, I, P]),
     "tw_latent_expand_store": (I, [I, P, L, P, I, I, P, P, I, I, I, I, I, I, I, P]),
     "tw_head_linear": (I, [I, P, L, I, P, P, L, I, I, I, I, I, P]),

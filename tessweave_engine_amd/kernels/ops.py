@@ -820,6 +820,43 @@ def latent_finish(proj, q_col, c_col, kr_col, cos, sin, norm_weight, q_out, head
                                      int(latent_dev), int(rot_dev), rot, page, float(eps), _stream()), "latent_finish")
 
 
+def latent_decode_splits(n_seqs, heads, max_kv_len):
+    return int(library().tw_latent_decode_splits(int(n_seqs), int(heads), int(max_kv_len)))
+
+
+def latent_decode_workspace_floats(n_seqs, heads, latent_dev, splits):
+    return int(library().tw_latent_decode_workspace_floats(int(n_seqs), int(heads), int(latent_dev), int(splits)))
+
+
+def latent_decode(q, keys, values, block_table, q_start, kv_len, n_seqs, out, heads, scale, splits=1, workspace=None):
+    """Attention of sequences 0 .. n_seqs - 1, ONE query token each, all heads against the one cached head: softmax of
+    scale * q_a . key over the sequence's keys, times the values (the first latent_dev elements of the key rows).
+    q [rows, heads * K] (head a at a * K), keys [pages, 1, page, K], values [pages, 1, latent_dev, page] (the same
+    elements, transposed inside a page), out [rows, heads * latent_dev]. splits > 1 cuts every sequence's keys into
+    ranges for separate workgroups; needs a float32 workspace of `latent_decode_workspace_floats` floats."""
+    page, K = keys.shape[2], keys.shape[3]
+    Lp = values.shape[2]
+    nq, wq, ldq = _rows(q, "q")
+    no, wo, ldo = _rows(out, "out")
+    _need(wq == heads * K and wo == heads * Lp and no >= n_seqs and nq >= n_seqs, "latent_decode q/out shapes do not agree")
+    _need(out.dtype == q.dtype == keys.dtype == values.dtype, "attention operand types differ")
+    _need(keys.dim() == 4 and keys.shape[1] == 1 and keys.is_contiguous() and values.is_contiguous()
+          and tuple(values.shape) == (keys.shape[0], 1, Lp, page), "keys [pages, 1, page, K], values [pages, 1, latent_dev, page]")
+    _need(K % 16 == 0 and K <= 256 and Lp % 16 == 0 and 16 <= Lp <= 240 and Lp <= K and page % 4 == 0, "unsupported sizes")
+    _need(block_table.dim() == 2 and block_table.stride(1) == 1 and block_table.shape[0] >= n_seqs, "block_table must be 2-D")
+    _need(q_start.numel() >= n_seqs + 1 and kv_len.numel() >= n_seqs, "sequence metadata is too short")
+    ws_ptr, ws_floats = None, 0
+    if splits > 1:
+        _need(workspace is not None and workspace.dtype == torch.float32, "split attention needs a float32 workspace")
+        ws_ptr, ws_floats = _dev(workspace), workspace.numel()
+    check(library().tw_latent_decode(dtype_id(q.dtype), _dev(q), ldq, _dev(keys), _dev(values),
+                                     _dev(block_table, torch.int32, "block_table"), block_table.stride(0),
+                                     _dev(q_start, torch.int32, "q_start"), _dev(kv_len, torch.int32, "kv_len"), int(n_seqs),
+                                     _dev(out), ldo, ws_ptr, ws_floats, int(heads), K, Lp, page, float(scale), int(splits),
+                                     _stream()), "latent_decode")
+    return out
+
+
 def latent_gather(keys, block_table, kv_len, kv_page_start, seq0, n_seqs, own_pages, rows, own_table):
     """The cached key rows of sequences seq0 .. seq0 + n_seqs - 1 from their pages into pages of their own, sequence after
     sequence (own page kv_page_start[s] - kv_page_start[seq0] + b holds block b of sequence s; places past a sequence's

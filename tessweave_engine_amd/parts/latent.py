@@ -48,8 +48,8 @@ class LatentAttention(Mixer):
         self.key_dev = self.latent_dev + self.rot_dev
         # the size of an expanded head (prompt portions): keys [unrotated | rotated] and values side by side in one size
         self.value_dev = self.head_dev = _round_up(max(self.dim + self.rot_dim, self.value_dim), 16)
-        if self.heads > 32 or self.key_dev > 256 or self.head_dev > 256:
-            raise ValueError("the attention kernels take up to 32 heads, latent + rotated sizes up to 256 and heads up to 256")
+        if self.key_dev > 256 or self.head_dev > 256:
+            raise ValueError("the attention kernels take latent + rotated sizes up to 256 and expanded heads up to 256")
         self.scale, self.eps, self.position, self.own_latent = float(scale), float(eps), position, bool(own_latent)
         self.proj = self.up = self.absorb = self.expand = self.latent_norm = None
         self.o = Linear([prefix + self.names[5]], heads * value_dim, [hidden], pad_in=(self.value_dim, self.value_dev),
@@ -137,14 +137,14 @@ class LatentAttention(Mixer):
             ops.head_linear(proj[:nd], self.dim_dev, self.absorb, q[:nd], K)
             mixed = ctx.scratch("latent.mixed", (n, H * Lp))[:nd]
             longest = ctx.kv_bound if ctx.capturing else ctx.max_kv_len
-            splits = ops.attn_mixed_splits(nd, longest)
+            splits = ops.latent_decode_splits(nd, H, longest)
             ws = None
             if splits > 1:
                 # sized for the most splits any length class can ask for, so that it never grows under a capture
-                floats = ops.attn_mixed_workspace_floats(nd, 1, H, Lp, max(splits, ops.attn_mixed_splits(nd, ctx.kv_capacity)))
-                ws = ctx.workspace.get("attn.mixed.split", (floats,), torch.float32)
-            ops.attn_mixed(q[:nd], keys, values, group.block_table, ctx.q_start, ctx.kv_len, 0, nd, 1, mixed, H, 1,
-                           self.scale, splits=splits, workspace=ws)
+                floats = ops.latent_decode_workspace_floats(nd, H, Lp, max(splits, ops.latent_decode_splits(nd, H, ctx.kv_capacity)))
+                ws = ctx.workspace.get("latent.split", (floats,), torch.float32)
+            ops.latent_decode(q[:nd], keys, values, group.block_table, ctx.q_start, ctx.kv_len, nd, mixed, H, self.scale,
+                              splits=splits, workspace=ws)
             ops.head_linear(mixed, Lp, self.expand, out[:nd], hd)
         if portions:
             # prompt portions: their sequences' cached latents expanded per head into pages of this step's own

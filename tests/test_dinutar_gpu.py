@@ -134,6 +134,55 @@ def test_head_linear(device, dtype, n, heads, n_in, n_out):
     assert (got[..., n_out:] == 7.0).all()
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("H,L,R,page,lengths,splits", [
+    (5, 48, 16, 4, [1, 7, 70], 1),             # fewer heads than a tile, pages of four keys, one key only
+    (20, 96, 32, 16, [300, 17, 1000], 0),      # two tiles of heads, key ranges as the launcher would choose them
+    (16, 192, 64, 16, [2049, 33], 9),          # ranges that get no key at all for the short sequence
+    (1, 16, 16, 8, [129], 3),
+])
+def test_one_token_attention_over_the_cached_latent(device, dtype, H, L, R, page, lengths, splits):
+    """All heads of a sequence against its one cached head: key rows [c | kr] on pages handed out in reverse order,
+    values = c once more, transposed inside a page; one key far back carries most of a head's weight; what lies in a
+    page behind a sequence's end is NaN and must not reach a sum."""
+    from tessweave_engine_amd.kernels import ops
+    dt = tdtype(dtype)
+    g = torch.Generator().manual_seed(L + R)
+    K, scale = L + R, 0.3
+    blocks = [(n + page - 1) // page for n in lengths]
+    n_pages = sum(blocks)
+    keys = torch.full((n_pages + 1, 1, page, K), float("nan"), dtype=dt)
+    values = torch.full((n_pages + 1, 1, L, page), float("nan"), dtype=dt)
+    table = torch.full((len(lengths), max(blocks)), -1, dtype=torch.int32)
+    q = (torch.randn(len(lengths), H, K, generator=g)).to(dt)
+    want, free = [], list(range(n_pages, 0, -1))
+    for s, n in enumerate(lengths):
+        rows = torch.randn(n, K, generator=g).to(dt)
+        far = n // 5
+        rows[far] = (q[s, 0].float() * 0.5).to(dt)                 # head 0 of this sequence looks at this key above all
+        for b in range(blocks[s]):
+            pg = free.pop(0)
+            table[s, b] = pg
+            part = rows[b * page:(b + 1) * page]
+            keys[pg, 0, :len(part)] = part
+            values[pg, 0, :, :len(part)] = part[:, :L].T
+        sc = torch.einsum("hk,nk->hn", q[s].double(), rows.double()) * scale
+        want.append(torch.softmax(sc, -1) @ rows[:, :L].double())
+    n_seqs = len(lengths)
+    if splits == 0:
+        splits = ops.latent_decode_splits(n_seqs, H, max(lengths))
+    floats = ops.latent_decode_workspace_floats(n_seqs, H, L, splits)
+    ws = torch.full((max(floats, 1),), float("nan"), device=device)
+    out = torch.zeros(n_seqs, H * L, dtype=dt, device=device)
+    ops.latent_decode(q.view(n_seqs, H * K).to(device), keys.to(device), values.to(device), table.to(device),
+                      ints(list(range(n_seqs + 1)), device), ints(lengths, device), n_seqs, out, H, scale, splits=splits,
+                      workspace=ws if floats else None)
+    got = out.cpu().double().view(n_seqs, H, L)
+    for s in range(n_seqs):
+        err = (got[s] - want[s]).abs().max().item()
+        assert err < (3e-2 if dtype == "bfloat16" else 2e-5), (s, err)
+
+
 def retention_case(H, D, E, rot_dims, decay, lengths, seed):
     """Raw projections [T, 2 H D + 2 H E] of several sequences and what the mechanism gives for each (float64)."""
     g = torch.Generator().manual_seed(seed)
