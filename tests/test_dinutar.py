@@ -133,3 +133,23 @@ def test_relu_squared():
     up = torch.tensor([[1.0, 0.0], [0.0, 1.0], [2.0, 0.0]], dtype=torch.float64)
     down = torch.tensor([[1.0, 1.0, 1.0]], dtype=torch.float64)
     assert plain.relu_squared_ff(h, up, down).item() == 1.0 + 0.0 + 4.0
+
+
+def test_command_line_inspect_and_random_weights(tmp_path, capsys):
+    """`random-weights` writes a folder for the design from its config.json alone; `inspect` reports the cache groups
+    (one key/value head of latent + rotated part, values of the latent's size) and what a request holds besides pages."""
+    from safetensors import safe_open
+    from tessweave_engine_amd.cli import main
+    c = CONFIGS["wide"]
+    (tmp_path / "config.json").write_text(json.dumps(c))
+    out = tmp_path / "model"
+    assert main(["random-weights", str(tmp_path / "config.json"), str(out), "--seed", "3"]) == 0
+    with safe_open(str(out / "model.safetensors"), framework="pt") as f:
+        assert {k: tuple(f.get_slice(k).get_shape()) for k in f.keys()} == tensor_shapes(c)
+    capsys.readouterr()
+    assert main(["inspect", str(out), "--kv-blocks", "10", "--block-size", "16"]) == 0
+    report = json.loads(capsys.readouterr().out)
+    groups = sorted((g["layers"], g["kv_heads"], g["head_dim"], g.get("value_dim")) for g in report["cache_groups"])
+    assert groups == [(1, 1, 48, 32), (1, 1, 128, 96)]
+    states = 4 * (1 * 64 * 128 + 4 * 16 * 16) + 4 * 2
+    assert report["state_bytes_per_request"] == states
