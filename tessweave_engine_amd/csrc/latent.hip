@@ -240,13 +240,39 @@ extern "C" int tw_latent_gather(int dtype, const void* keys, const int* block_ta
 }
 
 // One workgroup a page: up [rows][H * D + H * E] (the heads' key parts, then their value parts), kr at rows[row][Lp ..].
-template <typename T>
+// VEC (bfloat16, sizes and strides that are multiples of 8): 16 bytes a thread. A key row is copied in groups of 8
+// elements; for the transposed values a thread gathers one element of 8 consecutive places (neighbouring threads
+// read neighbouring elements of one row) and stores them as one group.
+template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void latent_expand_store_kernel(const T* __restrict__ up, long ld_up, const T* __restrict__ rows,
                                                                   int K, int Lp, T* __restrict__ keys, T* __restrict__ values,
                                                                   int H, int D, int R, int E, int hd, int P) {
   const int pg = blockIdx.x;
   T* kp = keys + (size_t)pg * H * P * hd;
   T* vp = values + (size_t)pg * H * hd * P;
+  if (VEC) {
+    const int groups = hd / 8;
+    for (int i = threadIdx.x; i < H * P * groups; i += blockDim.x) {
+      const int d = (i % groups) * 8, t = (i / groups) % P, a = i / (groups * P);
+      const size_t row = (size_t)pg * P + t;
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (d < D) v = *reinterpret_cast<const u32x4*>(up + row * ld_up + a * D + d);
+      else if (d < D + R) v = *reinterpret_cast<const u32x4*>(rows + row * K + Lp + d - D);
+      *reinterpret_cast<u32x4*>(kp + ((size_t)a * P + t) * hd + d) = v;
+    }
+    const int tgs = P / 8;
+    for (int i = threadIdx.x; i < H * tgs * hd; i += blockDim.x) {
+      const int e = i % hd, tg = (i / hd) % tgs, a = i / (hd * tgs);
+      bf16x8 v;
+#pragma unroll
+      for (int x = 0; x < 8; ++x) {
+        const size_t row = (size_t)pg * P + tg * 8 + x;
+        v[x] = e < E ? up[row * ld_up + (size_t)H * D + a * E + e] : (bf16_t)0.f;
+      }
+      *reinterpret_cast<bf16x8*>(vp + ((size_t)a * hd + e) * P + tg * 8) = v;
+    }
+    return;
+  }
   for (int i = threadIdx.x; i < H * P * hd; i += blockDim.x) {
     const int d = i % hd, t = (i / hd) % P, a = i / (hd * P);
     const size_t row = (size_t)pg * P + t;
@@ -268,12 +294,18 @@ extern "C" int tw_latent_expand_store(int dtype, const void* up, long ld_up, con
   TW_REQUIRE(up && rows && keys && values && own_pages >= 0 && H > 0 && D > 0 && R >= 0 && E > 0 && page_size > 0);
   TW_REQUIRE(hd >= D + R && hd >= E && ld_up >= (long)H * (D + E) && K >= Lp + R);
   if (own_pages == 0) return 0;
-  if (dtype == TW_DTYPE_BF16)
-    latent_expand_store_kernel<bf16_t><<<own_pages, 256, 0, stream>>>((const bf16_t*)up, ld_up, (const bf16_t*)rows, K, Lp,
-                                                                      (bf16_t*)keys, (bf16_t*)values, H, D, R, E, hd, page_size);
+  const bool vec = dtype == TW_DTYPE_BF16 && D % 8 == 0 && R % 8 == 0 && E % 8 == 0 && hd % 8 == 0 && page_size % 8 == 0 &&
+                   ld_up % 8 == 0 && K % 8 == 0 && Lp % 8 == 0 && (uintptr_t)up % 16 == 0 && (uintptr_t)rows % 16 == 0 &&
+                   (uintptr_t)keys % 16 == 0 && (uintptr_t)values % 16 == 0;
+  if (vec)
+    latent_expand_store_kernel<bf16_t, true><<<own_pages, 256, 0, stream>>>((const bf16_t*)up, ld_up, (const bf16_t*)rows, K, Lp,
+                                                                            (bf16_t*)keys, (bf16_t*)values, H, D, R, E, hd, page_size);
+  else if (dtype == TW_DTYPE_BF16)
+    latent_expand_store_kernel<bf16_t, false><<<own_pages, 256, 0, stream>>>((const bf16_t*)up, ld_up, (const bf16_t*)rows, K, Lp,
+                                                                             (bf16_t*)keys, (bf16_t*)values, H, D, R, E, hd, page_size);
   else if (dtype == TW_DTYPE_F32)
-    latent_expand_store_kernel<float><<<own_pages, 256, 0, stream>>>((const float*)up, ld_up, (const float*)rows, K, Lp,
-                                                                     (float*)keys, (float*)values, H, D, R, E, hd, page_size);
+    latent_expand_store_kernel<float, false><<<own_pages, 256, 0, stream>>>((const float*)up, ld_up, (const float*)rows, K, Lp,
+                                                                            (float*)keys, (float*)values, H, D, R, E, hd, page_size);
   else return TW_ERR_BAD_ARGUMENT;
   return TW_LAUNCH_RESULT();
 }

@@ -376,7 +376,7 @@ __global__ void retention_commit_kernel(RetentionArgs a, RetentionSegments sg, i
   const size_t count = (size_t)a.Dp * a.Ep;
   const float* src = sg.local + (((size_t)s_local * a.H + head) * sg.segments + (q_len - 1) / sg.seg_len) * count;
   float* dst = a.state + ((size_t)a.state_slots[s] * a.H + head) * count;
-  for (size_t i = threadIdx.x; i < count; i += blockDim.x) dst[i] = src[i];
+  for (size_t i = (size_t)blockIdx.y * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.y * blockDim.x) dst[i] = src[i];
 }
 
 static int retention_chunk_tokens(int Dp) { return Dp <= 128 ? 64 : 32; }
@@ -424,7 +424,7 @@ static int retention_chunk_launch_nt(const RetentionArgs& a, const RetentionSegm
   const dim3 grid((unsigned)n_seqs * a.H * slices, (unsigned)sg.segments);
   if (sg.segments > 1) retention_chunk_kernel<T, NT_MAX, EXACT, true><<<grid, 256, lds, stream>>>(a, sg, seq0, Bc);
   retention_chunk_kernel<T, NT_MAX, EXACT, false><<<grid, 256, lds, stream>>>(a, sg, seq0, Bc);
-  if (sg.segments > 1) retention_commit_kernel<<<dim3((unsigned)n_seqs * a.H), 256, 0, stream>>>(a, sg, seq0);
+  if (sg.segments > 1) retention_commit_kernel<<<dim3((unsigned)n_seqs * a.H, 32), 256, 0, stream>>>(a, sg, seq0);
   return TW_LAUNCH_RESULT();
 }
 

@@ -143,11 +143,31 @@ __global__ void relu_squared_kernel(T* __restrict__ x, long ld, int cols, long t
   *p = tw_from_float<T>(v * v);
 }
 
-extern "C" int tw_relu_squared(int dtype, void* x, long ld, int n, int cols, hipStream_t stream) {
-  TW_REQUIRE(x && n >= 0 && cols > 0 && ld >= cols);
+// The same from split-K partial sums of the product before (float32 [splits][n][cols], added in index order): one
+// rounding, and no kernel of its own for the sums.
+template <typename T>
+__global__ void relu_squared_sums_kernel(const float* __restrict__ partial, int splits, T* __restrict__ x, long ld, int cols,
+                                         long total) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  float v = 0.f;
+  for (int s = 0; s < splits; ++s) v += partial[(size_t)s * total + i];
+  v = fmaxf(v, 0.f);
+  x[(i / cols) * ld + i % cols] = tw_from_float<T>(v * v);
+}
+
+extern "C" int tw_relu_squared(int dtype, void* x, long ld, int n, int cols, const float* partial, int splits,
+                               hipStream_t stream) {
+  TW_REQUIRE(x && n >= 0 && cols > 0 && ld >= cols && (partial == nullptr || splits > 0));
   if (n == 0) return 0;
   const long total = (long)n * cols;
   const int blocks = tw_div_up(total, 256);
+  if (partial) {
+    if (dtype == TW_DTYPE_BF16) relu_squared_sums_kernel<bf16_t><<<blocks, 256, 0, stream>>>(partial, splits, (bf16_t*)x, ld, cols, total);
+    else if (dtype == TW_DTYPE_F32) relu_squared_sums_kernel<float><<<blocks, 256, 0, stream>>>(partial, splits, (float*)x, ld, cols, total);
+    else return TW_ERR_BAD_ARGUMENT;
+    return TW_LAUNCH_RESULT();
+  }
   if (dtype == TW_DTYPE_BF16) relu_squared_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)x, ld, cols, total);
   else if (dtype == TW_DTYPE_F32) relu_squared_kernel<float><<<blocks, 256, 0, stream>>>((float*)x, ld, cols, total);
   else return TW_ERR_BAD_ARGUMENT;

@@ -51,7 +51,7 @@ _SIGNATURES = {
     "tw_attn_mixed": (I, [I, P, L, P, P, P, I, P, P, I, I, I, P, L, P, P, P, P, L, I, I, I, I, I, I, F, F, I, P]),
     "tw_kv_store": (I, [I, P, L, I, I, P, P, P, I, I, I, I, I, P]),
     "tw_residual_norm": (I, [I, P, P, L, P, I, L, P, P, P, I, I, F, F, P]),
-    "tw_relu_squared": (I, [I, P, L, I, I, P]),
+    "tw_relu_squared": (I, [I, P, L, I, I, P, I, P]),
     "tw_embed_hashed": (I, [I, P, P, I, P, P, P, P, P, P, P, P, I, I, I, I, L, L, L, F, F, P, P, P]),
     "tw_latent_finish": (I, [I, P, L, I, I, I, P, P, P, P, L, P, L, I, I, I, I, P, P, P, I, I, I, I, I, I, I, F, P]),
     "tw_latent_decode_splits": (I, [I, I, I]),

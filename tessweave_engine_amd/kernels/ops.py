@@ -745,10 +745,17 @@ def residual_norm(x, weight, eps, out=None, y=None, add=None, scale=None, alpha=
     return x
 
 
-def relu_squared(x):
-    """x <- max(x, 0)^2 in place (rows may be strided)."""
+def relu_squared(x, partial=None):
+    """x <- max(x, 0)^2 in place (rows may be strided); with PARTIAL (float32 [splits, n, cols], split-K sums of the
+    product before) x <- max(sum of the splits, 0)^2 instead, rounded once."""
     n, cols, ld = _rows(x, "x")
-    check(library().tw_relu_squared(dtype_id(x.dtype), _dev(x), ld, n, cols, _stream()), "relu_squared")
+    splits = 0
+    if partial is not None:
+        _need(partial.dim() == 3 and partial.is_contiguous() and tuple(partial.shape[1:]) == (n, cols)
+              and partial.dtype == torch.float32, "partial sums must be float32 [splits, n, cols]")
+        splits = partial.shape[0]
+    check(library().tw_relu_squared(dtype_id(x.dtype), _dev(x), ld, n, cols, _dev(partial) if partial is not None else None,
+                                    splits, _stream()), "relu_squared")
     return x
 
 

@@ -108,8 +108,12 @@ class ReluSquaredFeedForward(FeedForward):
     def forward(self, ctx, h, x, accumulate=True):
         n = h.shape[0]
         act = ctx.scratch("ffn.act", (n, self.intermediate))
-        self.up.forward(ctx, h, act)
-        ops.relu_squared(act)
+        if n <= 64 and self.up.deferrable(n):
+            # few rows: the product leaves its split-K sums, and the activation's kernel adds them up
+            ops.relu_squared(act, partial=self.up.forward_partials(ctx, h, "up"))
+        else:
+            self.up.forward(ctx, h, act)
+            ops.relu_squared(act)
         if ctx.defer_sums and self.down.deferrable(n):
             return self.down.forward_partials(ctx, act, "down")          # whoever norms next adds them up
         self.down.forward(ctx, act, x, residual=x if accumulate else None)

@@ -277,6 +277,9 @@ def test_relu_squared_in_place(device):
     buf[:, :40] = x.to(device)
     ops.relu_squared(buf[:, :40])
     assert torch.equal(buf[:, :40].cpu(), (torch.relu(x.float()) ** 2).to(torch.bfloat16)) and (buf[:, 40:] == 0).all()
+    parts = torch.randn(3, 7, 40)
+    ops.relu_squared(buf[:, :40], partial=parts.to(device))
+    assert torch.equal(buf[:, :40].cpu(), (torch.relu(parts[0] + parts[1] + parts[2]) ** 2).to(torch.bfloat16)) and (buf[:, 40:] == 0).all()
 
 
 # ---------------------------------------------------------------------------------------------------------
