@@ -763,6 +763,19 @@ extern "C" int tw_linear(int dtype, int out_f32, const void* A, long lda, const 
   return TW_ERR_BAD_ARGUMENT;
 }
 
+// out = act(x @ W.T + bias) for many rows (the tiled kernels, whose epilogue and split-K reduction apply the
+// activation before the one rounding): more than 64 rows, K a multiple of 16 bytes, output in the input type.
+extern "C" int tw_linear_act(int dtype, const void* A, long lda, const void* W, long ldw, int shuffled, const float* bias,
+                             void* C, long ldc, float* partial, long partial_bytes, int M, int N, int K, int act,
+                             hipStream_t stream) {
+  TW_REQUIRE(act == TW_ACT_RELU_SQUARED);
+  TW_REQUIRE(M > 64 && N > 0 && K > 0 && lda >= K && ldc >= N && K % (dtype == TW_DTYPE_F32 ? 4 : 8) == 0);
+  TW_REQUIRE(dtype == TW_DTYPE_F32 || dtype == TW_DTYPE_BF16);
+  TW_REQUIRE(weight_layout_ok(dtype, shuffled, ldw, K));
+  return tw_tiled_linear(dtype, dtype == TW_DTYPE_F32 ? 1 : 0, shuffled, 0, 0, A, lda, W, ldw, bias, nullptr, (long)act, C, ldc,
+                         partial, partial_bytes, M, N, K, stream);
+}
+
 template <typename T>
 static int glu_layout(int shuffled, const T* A, long lda, const T* W, long ldw, const float* bias, T* C, long ldc,
                       int M, int N, int K, int force, long code, hipStream_t stream) {

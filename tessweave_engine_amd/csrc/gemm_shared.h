@@ -27,7 +27,19 @@ __device__ __forceinline__ float tw_glu(float g, float u, long code) {
   return factor * a * u;
 }
 
-// Sum of split-K partial sums partial[split][M][N], in split order, then bias and residual.
+// A plain product that adds no residual has the residual's row stride free as well: there it names an activation
+// of the result (after the bias, before the one rounding). 0: none; TW_ACT_RELU_SQUARED: max(x, 0)^2. Only the tiled
+// kernels (and the reduction of their split-K sums) read it: tw_linear_act is the entry point.
+#define TW_ACT_RELU_SQUARED 1
+__device__ __forceinline__ float tw_act(float x, long code) {
+  if (code == TW_ACT_RELU_SQUARED) {
+    x = fmaxf(x, 0.f);
+    return x * x;
+  }
+  return x;
+}
+
+// Sum of split-K partial sums partial[split][M][N], in split order, then bias and residual (or the activation).
 template <typename OutT>
 __global__ void splitk_reduce_kernel(const float* __restrict__ partial, int splits,
                                      const float* __restrict__ bias, const float* residual, long ldr,
@@ -39,6 +51,7 @@ __global__ void splitk_reduce_kernel(const float* __restrict__ partial, int spli
   for (int s = 0; s < splits; ++s) v += partial[(size_t)s * M * N + i];
   if (bias) v += bias[col];
   if (residual) v += residual[(size_t)row * ldr + col];
+  else v = tw_act(v, ldr);
   C[(size_t)row * ldc + col] = tw_from_float<OutT>(v);
 }
 
@@ -67,6 +80,10 @@ __global__ void splitk_reduce_vec4_kernel(const float* __restrict__ partial, int
   }
   if (bias) v = v + b;
   if (residual) v = v + r;
+  else if (ldr != 0) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = tw_act(v[e], ldr);
+  }
   OutT* dst = C + (size_t)row * ldc + col;
   if (sizeof(OutT) == 4) {
     *reinterpret_cast<f32x4*>(dst) = v;

@@ -120,6 +120,10 @@ __device__ __forceinline__ void tw_tiled_epilogue(f32x16 (&acc)[WM][WN], char* l
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] += lane_bias[t % NB][e];
       }
+      if (residual == nullptr && ldr != 0) {                 // (no residual: the stride names an activation, see tw_act)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = tw_act(v[e], ldr);
+      }
       if (vec_ok && col + 8 <= N) {
         if (residual) {
           const f32x4 r0 = *reinterpret_cast<const f32x4*>(residual + (size_t)row * ldr + col);

@@ -30,6 +30,7 @@ _SIGNATURES = {
     "tw_linear_partials": (I, [I, P, L, P, L, I, P, L, I, I, I, P]),
     "tw_linear_glu": (I, [I, P, L, P, L, I, P, P, L, I, I, I, I, I, F, P]),
     "tw_linear": (I, [I, I, P, L, P, L, I, P, P, L, P, L, P, L, I, I, I, I, P]),
+    "tw_linear_act": (I, [I, P, L, P, L, I, P, P, L, P, L, I, I, I, I, P]),
     "tw_attn_decode_splits": (I, [I, I, I, I]),
     "tw_attn_decode_workspace_floats": (L, [I, I, I, I]),
     "tw_attn_decode": (I, [I, P, L, P, P, P, I, P, P, I, I, P, L, P, L, I, I, I, I, I, F, F, I, I, P]),

@@ -339,6 +339,35 @@ def linear(x, weight, out, bias=None, residual=None, workspace=None, force=GEMM_
     return out
 
 
+LINEAR_ACTIVATIONS = {"relu_squared": 1}
+
+
+def can_linear_act(x, weight):
+    """Does `linear_act` take these operands? (more than 64 rows, K a multiple of 16 bytes: the tiled kernels)"""
+    k = weight.shape[1]
+    return x.shape[0] > 64 and k % (16 // x.element_size()) == 0
+
+
+def linear_act(x, weight, out, activation="relu_squared", bias=None, workspace=None):
+    """out = act(x @ weight.T + bias) in x's type, the activation applied in float32 in the matrix kernel's epilogue
+    (or where its split-K sums are added up) before the one rounding. For more than 64 rows (`can_linear_act`)."""
+    _need(activation in LINEAR_ACTIVATIONS, f"activation must be one of {sorted(LINEAR_ACTIVATIONS)}")
+    m, k, lda = _rows(x, "x")
+    n, k2, w_ptr, ldw, shuffled, w_dtype = _weight_args(weight)
+    mo, no, ldc = _rows(out, "out")
+    _need(k == k2 and mo == m and no == n, f"linear_act shapes do not agree: x {tuple(x.shape)}, weight {(n, k2)}, out {tuple(out.shape)}")
+    _need(x.dtype == w_dtype == out.dtype and can_linear_act(x, weight), "linear_act takes more than 64 rows of the weight's type")
+    if bias is not None:
+        _need(bias.numel() == n and bias.is_contiguous(), "bias has the wrong size")
+    ws_ptr, ws_bytes = None, 0
+    if workspace is not None:
+        ws_ptr, ws_bytes = _dev(workspace), workspace.numel() * workspace.element_size()
+    check(library().tw_linear_act(dtype_id(x.dtype), _dev(x), lda, w_ptr, ldw, shuffled,
+                                  _dev(bias, torch.float32, "bias") if bias is not None else None, _dev(out), ldc,
+                                  ws_ptr, ws_bytes, m, n, k, LINEAR_ACTIVATIONS[activation], _stream()), "linear_act")
+    return out
+
+
 def attn_decode_splits(n_seqs, q_heads, kv_heads, max_kv_len):
     return int(library().tw_attn_decode_splits(n_seqs, q_heads, kv_heads, max_kv_len))
 

@@ -111,7 +111,7 @@ class ReluSquaredFeedForward(FeedForward):
         if n <= 64 and self.up.deferrable(n):
             # few rows: the product leaves its split-K sums, and the activation's kernel adds them up
             ops.relu_squared(act, partial=self.up.forward_partials(ctx, h, "up"))
-        else:
+        elif not self.up.forward_act(ctx, h, act, "relu_squared"):       # many rows: in the product's epilogue
             self.up.forward(ctx, h, act)
             ops.relu_squared(act)
         if ctx.defer_sums and self.down.deferrable(n):

@@ -157,6 +157,17 @@ class Linear(Part):
         return ops.linear_glu(x, self.weights[0], out, bias=self.biases[0] if self.biases else None,
                               activation=activation, factor=factor)
 
+    def forward_act(self, ctx, x, out, activation):
+        """out = act(x @ W.T (+ bias)) in x's type, the activation in the matrix kernel's epilogue; True if it ran
+        (one packed matrix, more than 64 rows, K a multiple of 16 bytes), else nothing was written."""
+        if len(self.weights) != 1 or self.gated or not ops.can_linear_act(x, self.weights[0]):
+            return False
+        w = self.weights[0]
+        floats = ops.linear_workspace_bytes(w.dtype, x.shape[0], w.shape[0], w.shape[1]) // 4
+        ws = ctx.workspace.get("linear.splitk.rows", (floats,), torch.float32) if floats else None
+        ops.linear_act(x, w, out, activation, bias=self.biases[0] if self.biases else None, workspace=ws)
+        return True
+
     def forward(self, ctx, x, out, residual=None):
         """out[:, columns] = x @ W.T (+ bias) (+ residual); out may be float32 or x's type."""
         if self.gated:

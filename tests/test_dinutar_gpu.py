@@ -282,6 +282,27 @@ def test_relu_squared_in_place(device):
     assert torch.equal(buf[:, :40].cpu(), (torch.relu(parts[0] + parts[1] + parts[2]) ** 2).to(torch.bfloat16)) and (buf[:, 40:] == 0).all()
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("m,n,k,shuffled", [(65, 40, 96, True), (300, 272, 64, False), (2048, 1408, 512, True), (130, 4096, 2048, True)])
+def test_product_with_relu_squared_in_its_epilogue(device, dtype, m, n, k, shuffled):
+    """Against the product followed by the activation's own kernel (the same sums; one rounding instead of two), with
+    and without split-K sums, with a bias."""
+    from tessweave_engine_amd.kernels import ops
+    dt = tdtype(dtype)
+    g = torch.Generator().manual_seed(m + n)
+    x = torch.randn(m, k, generator=g).to(dt).to(device)
+    w = (torch.randn(n, k, generator=g) / math.sqrt(k)).to(dt).to(device)
+    bias = torch.randn(n, generator=g).to(device)
+    weight = ops.shuffle_weight(w) if shuffled else w
+    floats = ops.linear_workspace_bytes(dt, m, n, k) // 4
+    ws = torch.empty(max(floats, 1), device=device)
+    out = torch.empty(m, n, dtype=dt, device=device)
+    ops.linear_act(x, weight, out, "relu_squared", bias=bias, workspace=ws if floats else None)
+    want = torch.relu(x.double() @ w.double().T + bias.double()) ** 2
+    tol = 3e-2 if dtype == "bfloat16" else 1e-4
+    assert ((out.double() - want).abs() <= tol * (1 + want.abs())).all()
+
+
 # ---------------------------------------------------------------------------------------------------------
 # whole models
 # ---------------------------------------------------------------------------------------------------------
