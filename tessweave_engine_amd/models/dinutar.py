@@ -97,9 +97,8 @@ class DinutarConfig:
                     _positive(_need(m, key, where + "mixer."), f"layer {i}: {key}")
                 _need(m, "scale", where + "mixer.")
                 _check_rot(_need(m, "rot", where + "mixer."), m["rot_dim"], where + "mixer.rot.")
-                if (m["kv_rank"] + 15) // 16 * 16 + (m["rot_dim"] + 15) // 16 * 16 > 256 or max(m["dim"] + m["rot_dim"], m["vdim"]) > 256:
-                    raise ConfigError(f"layer {i}: the latent attention kernels take kv_rank + rot_dim (each rounded up to a "
-                                      "multiple of 16) up to 256, and dim + rot_dim and vdim up to 256")
+                if max(m["dim"] + m["rot_dim"], m["vdim"]) > 256:
+                    raise ConfigError(f"layer {i}: the attention kernels take dim + rot_dim and vdim up to 256")
                 source = m.get("kv_from")
                 if source is not None:
                     if isinstance(source, bool) or not isinstance(source, int) or not 0 <= source < i:

@@ -48,8 +48,14 @@ class LatentAttention(Mixer):
         self.key_dev = self.latent_dev + self.rot_dev
         # the size of an expanded head (prompt portions): keys [unrotated | rotated] and values side by side in one size
         self.value_dev = self.head_dev = _round_up(max(self.dim + self.rot_dim, self.value_dim), 16)
-        if self.key_dev > 256 or self.head_dev > 256:
-            raise ValueError("the attention kernels take latent + rotated sizes up to 256 and expanded heads up to 256")
+        if self.head_dev > 256:
+            raise ValueError("the attention kernels take expanded heads (dim + rot_dim, value_dim) up to 256")
+        # The one-head kernel of one-token sequences holds a key row's products in registers: latent + rotated part up
+        # to 256 elements. A larger latent sends one-token sequences the prompt portions' way (expanded per step: right,
+        # and slow; its scratch pages grow with the sequences, so such a model's steps are not replayed from graphs).
+        self.one_head = self.key_dev <= 256
+        if not self.one_head:
+            self.graph_safe = False
         self.scale, self.eps, self.position, self.own_latent = float(scale), float(eps), position, bool(own_latent)
         self.proj = self.up = self.absorb = self.expand = self.latent_norm = None
         self.o = Linear([prefix + self.names[5]], heads * value_dim, [hidden], pad_in=(self.value_dim, self.value_dev),
@@ -116,9 +122,11 @@ class LatentAttention(Mixer):
     def forward(self, ctx, run, h, x, accumulate=True):
         if run.writes_cache != self.own_latent:
             raise RuntimeError("a layer with a latent of its own writes its cache slot; one without reads another layer's")
-        n, H, nd = ctx.n_tokens, self.heads, ctx.n_decode
+        n, H = ctx.n_tokens, self.heads
+        nd = ctx.n_decode if self.one_head else 0          # sequences that take the one-head kernel
         Lp, Rp, K, hd = self.latent_dev, self.rot_dev, self.key_dev, self.head_dev
         portions = ctx.n_seqs - nd
+        longest_portion = max(ctx.max_q_len, 1)
         proj = ctx.scratch("latent.proj", (n, self.proj_width))
         self.proj.forward(ctx, h, proj)
         cos, sin = self.position.tables(ctx)
@@ -157,12 +165,12 @@ class LatentAttention(Mixer):
             own_keys = ctx.workspace.get("latent.keys", (own_pages, H, page, hd), ctx.dtype)
             own_values = ctx.workspace.get("latent.values", (own_pages, H, hd, page), ctx.dtype)
             ops.latent_expand_store(up, rows, Lp, own_keys, own_values, H, self.dim, self.rot_dim, self.value_dim)
-            split = ops.attn_prefill_split(portions, H, H, ctx.max_q_len, ctx.max_kv_len)
+            split = ops.attn_prefill_split(portions, H, H, longest_portion, ctx.max_kv_len)
             ws = None
             if split[0] > 1:
                 ws = ctx.workspace.get("attn.prefill_split", (ops.attn_prefill_workspace_floats(n, H, hd, split[0]),), torch.float32)
             ops.attn_prefill(q_full, own_keys, own_values, own_table, ctx.q_start, ctx.kv_len, nd,
-                             portions, ctx.max_q_len, out, H, H, hd, self.scale, split=split, workspace=ws)
+                             portions, longest_portion, out, H, H, hd, self.scale, split=split, workspace=ws)
         if ctx.defer_sums and self.o.deferrable(n):
             return self.o.forward_partials(ctx, out, "o")          # whoever norms next adds them up
         self.o.forward(ctx, out, x, residual=x if accumulate else None)

@@ -60,7 +60,14 @@ CONFIG_WIDE = config([retention(1, 64, 128, [1.0], 64, base=1e6, ff=192),
 CONFIG_ONE = config([latent(2, 16, 16, 32, 16, 0.25, base=20.0, scaling=(8.0, 8, 2.0, 1.0))],
                     width=48, vocab=97, alpha=2.5, scale=0.3, buckets=7, mul_prev=0, mul_cur=11)
 
-CONFIGS = {"odd": CONFIG_ODD, "wide": CONFIG_WIDE, "one": CONFIG_ONE}
+# a latent too large for the one-head kernel of one-token sequences (latent + rotated part over 256 elements): every
+# sequence then goes the prompt portions' way; read by a second layer
+CONFIG_DEEP = config([latent(2, 16, 16, 24, 272, 0.2, base=1000.0, ff=80),
+                      retention(2, 16, 16, [0.9, 0.99], 16),
+                      latent(3, 8, 16, 16, 272, 0.3, base=1000.0, kv_from=0)],
+                     width=64, vocab=120, alpha=1.2, scale=0.9, buckets=31, mul_prev=3, mul_cur=5)
+
+CONFIGS = {"odd": CONFIG_ODD, "wide": CONFIG_WIDE, "one": CONFIG_ONE, "deep": CONFIG_DEEP}
 
 
 def tensor_shapes(c):

@@ -307,7 +307,7 @@ def test_product_with_relu_squared_in_its_epilogue(device, dtype, m, n, k, shuff
 # whole models
 # ---------------------------------------------------------------------------------------------------------
 
-LENGTHS = {"odd": [61, 3, 40, 1, 29, 75], "wide": [50, 37, 2, 66], "one": [44, 9, 30]}
+LENGTHS = {"odd": [61, 3, 40, 1, 29, 75], "wide": [50, 37, 2, 66], "one": [44, 9, 30], "deep": [33, 5, 47]}
 
 
 @pytest.fixture(scope="module", params=list(CONFIGS))
@@ -380,7 +380,7 @@ def test_token_by_token(model, dtype, graphs):
     d = Driver(model["folder"], dtype, pages=24, page_size=4, graphs=graphs)
     got = d.run([[(rid, 1)] for _ in model["tokens"][rid]], model["tokens"])
     check_all(model, got, dtype, only=[rid])
-    if graphs:
+    if graphs and d.model.graph_safe_model:
         assert d.stepper.graph_replays > 0
     d.close()
 
