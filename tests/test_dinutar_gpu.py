@@ -489,6 +489,73 @@ def test_sharp_attention_over_a_long_prompt(device, tmp_path, dtype, name):
     d.close()
 
 
+def random_config(seed):
+    """A configuration drawn at random: layer kinds in any order, sizes that are mostly no multiples of 16, readers of
+    earlier latents, stretched and plain rotations, layers with and without a feed-forward."""
+    import random
+    from dinutar_util import config, latent, retention
+    rng = random.Random(seed)
+    even = lambda lo, hi: 2 * rng.randint(lo // 2, hi // 2)
+    layers, writers = [], []
+    for i in range(rng.randint(2, 6)):
+        ff = rng.choice([None, rng.randint(3, 20) * 8, rng.randint(20, 150)])
+        scaling = rng.choice([None, (rng.choice([2.0, 4.0, 16.0]), rng.choice([8, 32, 100]), rng.choice([4.0, 32.0]), rng.choice([0.5, 1.0]))])
+        if rng.random() < 0.55 or i == 0 and rng.random() < 0.5:
+            if writers and rng.random() < 0.4:
+                j = rng.choice(writers)
+                m = layers[j]["mixer"]
+                lay = latent(rng.randint(1, 19), even(2, 60), m["rot_dim"], rng.randint(1, 70), m["kv_rank"], rng.uniform(0.05, 0.4), kv_from=j, ff=ff)
+                lay["mixer"]["rot"] = m["rot"]
+            else:
+                rot_dim = even(2, 40)
+                lay = latent(rng.randint(1, 19), even(2, 60), rot_dim, rng.randint(1, 70), rng.randint(4, 150), rng.uniform(0.05, 0.4),
+                             base=rng.choice([50.0, 1e4, 1e6]), scaling=scaling, ff=ff)
+                writers.append(i)
+        else:
+            heads, dim = rng.randint(1, 5), even(2, 70)
+            lay = retention(heads, dim, rng.randint(1, 150), [rng.choice([1.0, rng.uniform(0.3, 0.9999)]) for _ in range(heads)],
+                            even(2, dim), base=rng.choice([30.0, 1e4]), scaling=scaling, ff=ff)
+        layers.append(lay)
+    return config(layers, width=rng.choice([40, 56, 100, 136, 192]), vocab=rng.randint(30, 400), alpha=rng.choice([1.0, 0.7, 2.2]),
+                  scale=rng.uniform(0.3, 2.0), buckets=rng.randint(3, 5000), mul_prev=rng.randint(0, 10 ** 6), mul_cur=rng.randint(0, 10 ** 6),
+                  eps=rng.choice([1e-6, 1e-5, 1e-3]))
+
+
+@pytest.mark.parametrize("seed", list(range(8)))
+def test_configurations_drawn_at_random(device, tmp_path, seed):
+    """Whole prompts in one batch, then a prompt in portions with its last tokens one by one beside another request, in
+    both precisions, for sizes nobody chose."""
+    c = random_config(seed)
+    weights = make_weights(c, seed=100 + seed)
+    folder = write_folder(tmp_path, c, weights)
+    g = torch.Generator().manual_seed(seed)
+    tokens = {"a": torch.randint(0, c["vocab"], (83,), generator=g).tolist(), "b": torch.randint(0, c["vocab"], (21,), generator=g).tolist()}
+    want = {k: plain.forward(c, weights, v).numpy() for k, v in tokens.items()}
+    for dtype in ("float32", "bfloat16"):
+        d = Driver(folder, dtype, pages=40, page_size=4, max_requests=2)
+        whole = d.run([[("a", 83), ("b", 21)]], tokens)
+        cut = d.run([[("a", 30)], [("a", 17), ("b", 2)], [("a", 2), ("b", 1)], [("a", 24), ("b", 9)]] + [[("a", 1), ("b", 1)]] * 10, tokens)
+        for got in (whole, cut):
+            check_rows(np.concatenate([row_error(got[k], want[k]) for k in tokens]), dtype, (seed, c["width"]))
+        d.close()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_prompt_in_one_step(device, tmp_path, dtype):
+    """1,700 tokens: 1,500 in one step (retention in several segments a sequence, prompt attention over many tiles),
+    then a portion of 150 behind them and single tokens, beside a second, short request."""
+    c = CONFIGS["odd"]
+    weights = make_weights(c, seed=17)
+    folder = write_folder(tmp_path, c, weights)
+    g = torch.Generator().manual_seed(6)
+    tokens = {"a": torch.randint(0, c["vocab"], (1700,), generator=g).tolist(), "b": torch.randint(0, c["vocab"], (40,), generator=g).tolist()}
+    want = {k: plain.forward(c, weights, v).numpy() for k, v in tokens.items()}
+    d = Driver(folder, dtype, pages=120, page_size=16, max_requests=2)
+    got = d.run([[("a", 1500), ("b", 3)], [("a", 150), ("b", 1)]] + [[("a", 1), ("b", 1)]] * 36 + [[("a", 14)]], tokens)
+    check_rows(np.concatenate([row_error(got[k], want[k]) for k in tokens]), dtype)
+    d.close()
+
+
 def test_long_decoding_from_graphs(device, tmp_path):
     """400 tokens decoded one by one from graphs after a short prompt, two requests side by side."""
     c = CONFIGS["odd"]
