@@ -102,8 +102,8 @@ static int retention_walk_launch(const RetentionArgs& a, int seq0, int n_seqs, h
 }
 
 // Portions of prompts: a workgroup owns 64 value columns of one (sequence, head, segment of the portion) and walks its
-// segment in chunks of Bc tokens (64, or 32 for long keys). Per chunk, with i, j the tokens' places in it, n its tokens
-// and g the decay:
+// segment in chunks of Bc tokens (32; 64 for keys of up to 64 elements: what keeps a workgroup's LDS under a third
+// of a CU's). Per chunk, with i, j the tokens' places in it, n its tokens and g the decay:
 //
 //   P^T[j][i] = g^(i - j) k_j . q_i  (j <= i)            the waves share the 16 x 16 tiles out; through LDS to all
 //   O^T[e][i] = sum_j V^T[e][j] P^T[j][i] + g^(i + 1) sum_d S[d][e] q_i[d]       wave w: columns 16 w .. of the slice
@@ -379,7 +379,7 @@ __global__ void retention_commit_kernel(RetentionArgs a, RetentionSegments sg, i
   for (size_t i = (size_t)blockIdx.y * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.y * blockDim.x) dst[i] = src[i];
 }
 
-static int retention_chunk_tokens(int Dp) { return Dp <= 128 ? 64 : 32; }
+static int retention_chunk_tokens(int Dp) { return Dp <= 64 ? 64 : 32; }
 
 static size_t retention_chunk_lds(int Dp, int Bc) {
   return ((size_t)2 * Bc * (Dp + 4) + (size_t)Bc * 68 + (size_t)Bc * (Bc + 4) + Bc) * sizeof(float);
@@ -391,7 +391,7 @@ static void retention_segments(int n_seqs, int max_q_len, int H, int Dp, int Ep,
   const int Bc = retention_chunk_tokens(Dp);
   const int chunks = tw_div_up(max_q_len, Bc);
   const long groups = (long)n_seqs * H * ((Ep + 63) / 64);
-  long want = tw_div_up(512, groups);
+  long want = tw_div_up(1024, groups);
   if (want > chunks / 4) want = chunks / 4;
   if (want < 1) want = 1;
   const int per = tw_div_up(chunks, want);
